@@ -19,7 +19,7 @@
 namespace tinyinfer {
 
 bool CacheNeed::operator==(const CacheNeed& o) const {
-  return kind == o.kind && kv_heads == o.kv_heads && head_dim == o.head_dim && window == o.window &&
+  return kind == o.kind && kv_heads == o.kv_heads && head_dim == o.head_dim && value_dim() == o.value_dim() && window == o.window &&
          state_shape == o.state_shape && row_shape == o.row_shape && rows_f32 == o.rows_f32;
 }
 

@@ -392,6 +392,7 @@ void ensure_builtin_architectures() {
     const ConfigReader typed = [](const Json& config) { return Qwen3Config::from_json(config).to_json(); };
     architectures().push_back({"Qwen3ForCausalLM", build_qwen3_spec, typed});
     architectures().push_back({"qwen3", build_qwen3_spec, typed});
+    architectures().push_back({"Miterax", miterax_spec, miterax_typed_config});
   });
 }
 
@@ -403,6 +404,8 @@ std::vector<std::string> candidates(const Json& config) {
         if (v.type() == Json::String) c.push_back(v.as_string());
   if (const Json* m = config.find("model_type"))
     if (m->type() == Json::String) c.push_back(m->as_string());
+  if (const Json* a = config.find("architecture"))       // some config.json files name their one architecture so
+    if (a->type() == Json::String) c.push_back(a->as_string());
   return c;
 }
 
@@ -451,7 +454,7 @@ Architecture architecture_of(const Json& config) {
   ensure_builtin_architectures();
   const auto cand = candidates(config);
   if (cand.empty())
-    throw ConfigError("config.json: neither 'architectures' nor 'model_type' names the model; registered: " +
+    throw ConfigError("config.json: neither 'architectures', 'model_type' nor 'architecture' names the model; registered: " +
                       list_of(registered_architectures()));
   {
     std::lock_guard<std::mutex> lock(g_arch_mutex);

@@ -126,3 +126,131 @@ extern "C" int ti_attention_rows(int dtype, const void* q, const void* pool, con
   TI_LAUNCH_CHECK();
   return 0;
 }
+
+// ------------------------------------------------------------------------------------------------
+// The same walk for attention whose keys and values differ in size and whose scores are soft-capped:
+//   s = (q . k) * scale;  s <- softcap * tanh(s / softcap)  (softcap <= 0: none);  softmax over the
+// visible keys.  Any key size dk and value size dv up to 256 (lanes beyond a size idle).  A page is
+// K [n_kv][P][dk] | V [n_kv][dv][P]; with dk == dv that is the layout above.
+template <typename T, int DPL>
+__global__ void __launch_bounds__(256)
+attention_capped_kernel(const T* __restrict__ q, const T* __restrict__ pool, const int* __restrict__ table,
+                        int table_stride, const int* __restrict__ pos, const int* __restrict__ slot,
+                        T* __restrict__ out, int n_head, int n_kv, int dk, int dv, int P, float scale, float softcap,
+                        int window) {
+  constexpr int HD = DPL * AG_LANES;
+  __shared__ float s_o[AG_GROUPS][HD];
+  __shared__ float s_m[AG_GROUPS], s_l[AG_GROUPS];
+  const int m = blockIdx.x, h = blockIdx.y;
+  const int g = threadIdx.x / AG_LANES, lane = threadIdx.x % AG_LANES;
+  const int kvh = h / (n_head / n_kv);
+  const int p_q = pos[m];
+  const int lo = (window > 0 && p_q - window + 1 > 0) ? p_q - window + 1 : 0;
+  const int* tab = table + (size_t)slot[m] * table_stride;
+  const size_t page_elems = (size_t)n_kv * P * (dk + dv);
+  const size_t k_off = (size_t)kvh * P * dk;
+  const size_t v_off = (size_t)n_kv * P * dk + (size_t)kvh * dv * P;
+  const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
+
+  float qv[DPL], o[DPL];
+  const T* qh = q + ((size_t)m * n_head + h) * dk;
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) {
+    const int d = lane + i * AG_LANES;
+    qv[i] = d < dk ? ld<T>(qh + d) : 0.f;
+    o[i] = 0.f;
+  }
+  float mx = -INFINITY, l = 0.f;
+  for (int p = lo + g; p <= p_q; p += AG_GROUPS) {
+    const int page = tab[p / P];
+    if (page < 0) continue;
+    const T* kp = pool + (size_t)page * page_elems + k_off + (size_t)(p % P) * dk;
+    const T* vp = pool + (size_t)page * page_elems + v_off + (p % P);
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) {
+      const int d = lane + i * AG_LANES;
+      if (d < dk) s = fmaf(qv[i], ld<T>(kp + d), s);
+    }
+    s = group_sum<AG_LANES>(s) * scale;
+    if (softcap > 0.f) s = softcap * tanhf(s * inv_cap);
+    const float m_new = fmaxf(mx, s);
+    const float alpha = expf(mx - m_new);
+    const float w = expf(s - m_new);
+    l = l * alpha + w;
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) {
+      const int d = lane + i * AG_LANES;
+      if (d < dv) o[i] = o[i] * alpha + w * ld<T>(vp + (size_t)d * P);
+    }
+    mx = m_new;
+  }
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) s_o[g][lane + i * AG_LANES] = o[i];
+  if (lane == 0) {
+    s_m[g] = mx;
+    s_l[g] = l;
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < dv; d += 256) {
+    float mm = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < AG_GROUPS; ++j) mm = fmaxf(mm, s_m[j]);
+    float lt = 0.f, acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < AG_GROUPS; ++j) {
+      const float w = (s_m[j] == -INFINITY) ? 0.f : expf(s_m[j] - mm);
+      lt += s_l[j] * w;
+      acc += s_o[j][d] * w;
+    }
+    st<T>(out + ((size_t)m * n_head + h) * dv + d, acc / lt);
+  }
+}
+
+template <typename T>
+static int launch_capped(int dpl, dim3 grid, const void* q, const void* pool, const int* table, int table_stride,
+                         const int* pos, const int* slot, void* out, int n_head, int n_kv, int dk, int dv, int P,
+                         float scale, float softcap, int window, hipStream_t stream) {
+#define AG_CASE(D)                                                                                              \
+  case D:                                                                                                       \
+    attention_capped_kernel<T, D><<<grid, 256, 0, stream>>>((const T*)q, (const T*)pool, table, table_stride, pos, \
+                                                            slot, (T*)out, n_head, n_kv, dk, dv, P, scale, softcap, \
+                                                            window);                                            \
+    break;
+  switch (dpl) {
+    AG_CASE(1) AG_CASE(2) AG_CASE(3) AG_CASE(4) AG_CASE(5) AG_CASE(6) AG_CASE(7) AG_CASE(8)
+    AG_CASE(9) AG_CASE(10) AG_CASE(11) AG_CASE(12) AG_CASE(13) AG_CASE(14) AG_CASE(15) AG_CASE(16)
+    default:
+      return 1;
+  }
+#undef AG_CASE
+  return 0;
+}
+
+// q: [M, n_head, dk], out: [M, n_head, dv] in T; pool: [pages][K: [n_kv][P][dk] | V: [n_kv][dv][P]] in T
+extern "C" int ti_attention_capped_rows(int dtype, const void* q, const void* pool, const int* table, int table_stride,
+                                        const int* pos, const int* slot, void* out, int M, int n_head, int n_kv, int dk,
+                                        int dv, int page_size, float scale, float softcap, int window,
+                                        hipStream_t stream) {
+  TI_REQUIRE(dk >= 1 && dk <= 256 && dv >= 1 && dv <= 256, "attention: key size %d / value size %d are not served (up to 256)",
+             dk, dv);
+  TI_REQUIRE(n_head > 0 && n_kv > 0 && n_head % n_kv == 0, "attention: heads %d / kv_heads %d", n_head, n_kv);
+  TI_REQUIRE(n_head <= 65535, "attention: too many heads (%d)", n_head);
+  TI_REQUIRE(page_size > 0 && table_stride > 0, "attention: bad page_size %d / table_stride %d", page_size, table_stride);
+  if (M == 0) return 0;
+  dim3 grid(M, n_head);
+  const int big = dk > dv ? dk : dv;
+  const int dpl = (big + AG_LANES - 1) / AG_LANES;
+  int rc;
+  if (dtype == TI_F32)
+    rc = launch_capped<float>(dpl, grid, q, pool, table, table_stride, pos, slot, out, n_head, n_kv, dk, dv, page_size, scale,
+                              softcap, window, stream);
+  else if (dtype == TI_BF16)
+    rc = launch_capped<bf16_t>(dpl, grid, q, pool, table, table_stride, pos, slot, out, n_head, n_kv, dk, dv, page_size, scale,
+                               softcap, window, stream);
+  else
+    TI_REQUIRE(false, "attention: unknown dtype %d", dtype);
+  TI_REQUIRE(rc == 0, "attention: no kernel for sizes %d / %d", dk, dv);
+  TI_LAUNCH_CHECK();
+  return 0;
+}

@@ -58,7 +58,7 @@ def libraries_for(dtype: str) -> List[str]:
 # the host library (configuration, weights, parts, cache manager, step function, scheduler, sampler
 # and the C interface the Python package binds): C++17, no device code
 PKG = os.path.dirname(HERE)
-HOST_SOURCES = ["config/json.cpp", "config/config.cpp", "ops/ops.cpp", "parts/parts.cpp", "weights/weights.cpp",
+HOST_SOURCES = ["config/json.cpp", "config/config.cpp", "config/miterax.cpp", "ops/ops.cpp", "parts/parts.cpp", "weights/weights.cpp",
                 "models/model.cpp", "cache/cache_manager.cpp", "engine/engine.cpp", "engine/scheduler.cpp",
                 "sampling/sampler.cpp", "engine/c_api.cpp"]
 HOST_HEADERS = ["include/inference.h", "weights/weights.h", "csrc/tinyinfer_kernels.h"]

@@ -1,0 +1,144 @@
+// Element-wise kernels of layers that are not the plain pre-norm transformer block: an additive
+// sinusoidal position vector, a learned vector added to every row, the xIELU activation between the
+// two products of a dense feed-forward, the per-channel scaled sum of a parallel block's branches
+// into the residual, and the split of a fused q/k/v projection (keys and values of different sizes,
+// a position-dependent factor on the query) into the paged cache.  All arithmetic is 32-bit; T is
+// the storage type of activations and cache.
+#include "common.h"
+#include "tinyinfer_kernels.h"
+
+TI_ERROR_API
+
+// ------------------------------------------------------------ sinusoidal positions
+// x[m, 2i] += sin(pos[m] * inv_freq[i]),  x[m, 2i + 1] += cos(pos[m] * inv_freq[i])
+__global__ void add_sinusoid_kernel(float* __restrict__ x, const int* __restrict__ pos,
+                                    const float* __restrict__ inv_freq, int H) {
+  const int m = blockIdx.x;
+  const float p = (float)pos[m];
+  float* row = x + (size_t)m * H;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    const float a = p * inv_freq[c >> 1];
+    row[c] += (c & 1) ? cosf(a) : sinf(a);
+  }
+}
+
+extern "C" int ti_add_sinusoid(float* x, const int* pos, const float* inv_freq, int M, int H, hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && H > 0, "add_sinusoid: bad sizes M=%d H=%d", M, H);
+  if (M == 0) return 0;
+  add_sinusoid_kernel<<<M, 256, 0, stream>>>(x, pos, inv_freq, H);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------ one vector onto every row
+__global__ void add_row_kernel(float* __restrict__ x, const float* __restrict__ v, long n, int H) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) x[i] += v[i % H];
+}
+
+extern "C" int ti_add_row(float* x, const float* v, int M, int H, hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && H > 0, "add_row: bad sizes M=%d H=%d", M, H);
+  if (M == 0) return 0;
+  const long n = (long)M * H;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+  add_row_kernel<<<blocks, 256, 0, stream>>>(x, v, n, H);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------ xIELU
+// act = (p, q), two learned numbers.  z > 0: softplus(p) z^2 + z / 2;  z <= 0: (1/2 + softplus(q))
+// (exp(z) - 1 - z) + z / 2.
+__device__ __forceinline__ float softplus_f(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
+__device__ __forceinline__ float xielu_f(float z, float ap, float an) {
+  return z > 0.f ? fmaf(ap * z, z, 0.5f * z) : fmaf(an, expm1f(z) - z, 0.5f * z);
+}
+
+template <typename T>
+__global__ void xielu_kernel(const float* __restrict__ z, const float* __restrict__ act, T* __restrict__ out, long n) {
+  const float ap = softplus_f(act[0]), an = 0.5f + softplus_f(act[1]);
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+    st<T>(out + i, xielu_f(z[i], ap, an));
+}
+
+extern "C" int ti_xielu(int out_dtype, const float* z, const float* act, void* out, long n, hipStream_t stream) {
+  TI_REQUIRE(n >= 0, "xielu: bad count %ld", n);
+  if (n == 0) return 0;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+  if (out_dtype == TI_F32) xielu_kernel<float><<<blocks, 256, 0, stream>>>(z, act, (float*)out, n);
+  else if (out_dtype == TI_BF16) xielu_kernel<bf16_t><<<blocks, 256, 0, stream>>>(z, act, (bf16_t*)out, n);
+  else TI_REQUIRE(false, "xielu: unknown dtype %d", out_dtype);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------ scaled sum into the residual
+// x[m, c] += a[m, c] * sa[c] + b[m, c] * sb[c]   (b may be null: one branch; a scale that is null is 1)
+__global__ void scaled_add_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ sa,
+                                  const float* __restrict__ b, const float* __restrict__ sb, long n, int H) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const int c = (int)(i % H);
+    float y = a[i] * (sa ? sa[c] : 1.f);
+    if (b) y = fmaf(b[i], sb ? sb[c] : 1.f, y);
+    x[i] += y;
+  }
+}
+
+extern "C" int ti_scaled_add(float* x, const float* a, const float* sa, const float* b, const float* sb, int M, int H,
+                             hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && H > 0 && a, "scaled_add: bad sizes M=%d H=%d", M, H);
+  if (M == 0) return 0;
+  const long n = (long)M * H;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+  scaled_add_kernel<<<blocks, 256, 0, stream>>>(x, a, sa, b, sb, n, H);
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------ q/k/v split with a query temperature
+// qkv f32 [M, n_head dk + n_kv dk + n_kv dv].  q[m] times 1 + coef ln(floor((pos + 1) / every) + 1)
+// goes to q_out (T) [M, n_head dk]; k and v into the page of the token's position,
+// page = table[slot][pos / P], a page being  K [n_kv][P][dk] | V [n_kv][dv][P]  (values transposed).
+template <typename T>
+__global__ void qkv_split_write_kernel(const float* __restrict__ qkv, const int* __restrict__ pos,
+                                       const int* __restrict__ slot, const int* __restrict__ table, int table_stride,
+                                       T* __restrict__ pool, T* __restrict__ q_out, int n_head, int n_kv, int dk, int dv,
+                                       int P, float coef, int every) {
+  const int m = blockIdx.x;
+  const int p = pos[m];
+  const int nq = n_head * dk, nk = n_kv * dk, nv = n_kv * dv;
+  const float* row = qkv + (size_t)m * (nq + nk + nv);
+  const float temp = (coef != 0.f && every > 0) ? 1.f + coef * logf((float)((p + 1) / every) + 1.f) : 1.f;
+  for (int e = threadIdx.x; e < nq; e += blockDim.x) st<T>(q_out + (size_t)m * nq + e, row[e] * temp);
+  const int page = table[(size_t)slot[m] * table_stride + p / P];
+  if (page < 0) return;   // the host reserves pages first; never write astray
+  const int r = p % P;
+  T* base = pool + (size_t)page * ((size_t)n_kv * P * (dk + dv));
+  for (int e = threadIdx.x; e < nk; e += blockDim.x) {
+    const int h = e / dk, d = e % dk;
+    st<T>(base + ((size_t)h * P + r) * dk + d, row[nq + e]);
+  }
+  T* vbase = base + (size_t)n_kv * P * dk;
+  for (int e = threadIdx.x; e < nv; e += blockDim.x) {
+    const int h = e / dv, d = e % dv;
+    st<T>(vbase + ((size_t)h * dv + d) * P + r, row[nq + nk + e]);
+  }
+}
+
+extern "C" int ti_qkv_split_write(int dtype, const float* qkv, const int* pos, const int* slot, const int* table,
+                                  int table_stride, void* pool, void* q_out, int M, int n_head, int n_kv, int dk, int dv,
+                                  int page_size, float coef, int every, hipStream_t stream) {
+  TI_REQUIRE(n_head > 0 && n_kv > 0 && dk > 0 && dv > 0 && page_size > 0 && table_stride > 0,
+             "qkv_split_write: bad sizes heads=%d kv_heads=%d dk=%d dv=%d page=%d table_stride=%d", n_head, n_kv, dk, dv,
+             page_size, table_stride);
+  if (M == 0) return 0;
+  if (dtype == TI_F32)
+    qkv_split_write_kernel<float><<<M, 256, 0, stream>>>(qkv, pos, slot, table, table_stride, (float*)pool, (float*)q_out,
+                                                         n_head, n_kv, dk, dv, page_size, coef, every);
+  else if (dtype == TI_BF16)
+    qkv_split_write_kernel<bf16_t><<<M, 256, 0, stream>>>(qkv, pos, slot, table, table_stride, (bf16_t*)pool,
+                                                          (bf16_t*)q_out, n_head, n_kv, dk, dv, page_size, coef, every);
+  else
+    TI_REQUIRE(false, "qkv_split_write: unknown dtype %d", dtype);
+  TI_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,194 @@
+// Recurrent mixers: the mLSTM cell (a matrix memory per head with a stabilised exponential input
+// gate), as a scan over the tokens each request brings to a step, from and into the request's state.
+//
+// Per head, with keys k (dk), values v (dv), a log input gate i and a log forget gate f:
+//   m_t = max(f_t + m_(t-1), i_t)
+//   S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T        (dk x dv)
+//   n_t = the same with k_t alone                                            (dk)
+//   o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6)
+// The gates come from pre-activations a (with a bias b): i = cap tanh((a_i + b_i) / cap),
+// f = logsigmoid(cap tanh((a_f + b_f) / cap)).  State, gates and everything else here is 32-bit.
+//
+// One workgroup per (request of the step, head).  A wavefront owns 16 columns of S; the four lanes
+// that share a column hold a quarter of its rows each, in registers, for all tokens of the step.  The
+// tokens' q, k, v and gates pass through LDS sixteen at a time.  Every element of S, n and o is
+// computed by the same sequence of operations whether its token came alone or in a portion, so a
+// sequence cut differently gives the same bits.
+#include "common.h"
+#include "tinyinfer_kernels.h"
+
+TI_ERROR_API
+
+#define ML_COLS 16   // columns of the memory per wavefront
+#define ML_RG 4      // lanes sharing a column
+#define ML_TB 16     // tokens staged at a time
+
+__device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+template <int RPL, int MAXT>
+__global__ void __launch_bounds__(MAXT)
+mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, int off_v, int off_i, int off_f,
+                  const float* __restrict__ bias_i, const float* __restrict__ bias_f, float* __restrict__ state,
+                  long slot_stride, const int* __restrict__ entries, float* __restrict__ o, int heads, int dk, int dv,
+                  float cap, float q_scale) {
+  constexpr int DP = RPL * ML_RG;   // rows, padded
+  extern __shared__ __align__(16) float lds[];
+  float* lq = lds;                        // [ML_TB][DP]
+  float* lk = lq + ML_TB * DP;            // [ML_TB][DP]
+  float* lv = lk + ML_TB * DP;            // [ML_TB][dv]
+  float* lgi = lv + ML_TB * dv;           // [ML_TB]
+  float* lgf = lgi + ML_TB;               // [ML_TB]
+  const int e = blockIdx.x, h = blockIdx.y;
+  const int row0 = entries[4 * e], n_tok = entries[4 * e + 1], slot = entries[4 * e + 3];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, rg = lane >> 4, c = lane & 15;
+  const int n_waves = blockDim.x >> 6;
+  float* S_base = state + (size_t)slot * slot_stride + (size_t)h * ((size_t)dk * dv + dk + 1);
+  float* n_base = S_base + (size_t)dk * dv;
+  float* m_ptr = n_base + dk;
+  const int ov = heads * dv;
+  const int span = n_waves * ML_COLS;
+  float S[RPL], nn[RPL];
+  float m = 0.f;
+  for (int j0 = 0; j0 < dv; j0 += span) {
+    const int j = j0 + wave * ML_COLS + c;
+    const bool active = j < dv;
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+      const int r = rg * RPL + i;
+      S[i] = (active && r < dk) ? S_base[(size_t)r * dv + j] : 0.f;
+      nn[i] = r < dk ? n_base[r] : 0.f;
+    }
+    m = *m_ptr;
+    for (int t0 = 0; t0 < n_tok; t0 += ML_TB) {
+      const int tb = n_tok - t0 < ML_TB ? n_tok - t0 : ML_TB;
+      __syncthreads();   // the reads of the tokens before are over
+      for (int idx = threadIdx.x; idx < tb * DP; idx += blockDim.x) {
+        const int t = idx / DP, r = idx % DP;
+        const float* row = proj + (size_t)(row0 + t0 + t) * ld;
+        lq[idx] = r < dk ? row[off_q + h * dk + r] * q_scale : 0.f;
+        lk[idx] = r < dk ? row[off_k + h * dk + r] : 0.f;
+      }
+      for (int idx = threadIdx.x; idx < tb * dv; idx += blockDim.x) {
+        const int t = idx / dv, jj = idx % dv;
+        lv[idx] = proj[(size_t)(row0 + t0 + t) * ld + off_v + h * dv + jj];
+      }
+      if ((int)threadIdx.x < tb) {
+        const float* row = proj + (size_t)(row0 + t0 + threadIdx.x) * ld;
+        const float ai = row[off_i + h] + bias_i[h], af = row[off_f + h] + bias_f[h];
+        lgi[threadIdx.x] = cap * tanhf(ai / cap);
+        lgf[threadIdx.x] = log_sigmoid_f(cap * tanhf(af / cap));
+      }
+      __syncthreads();
+      for (int t = 0; t < tb; ++t) {
+        const float ig = lgi[t], fg = lgf[t];
+        const float m_new = fmaxf(fg + m, ig);
+        const float decay = expf(fg + m - m_new), take = expf(ig - m_new);
+        m = m_new;
+        const float tv = active ? take * lv[t * dv + j] : 0.f;
+        const float4* q4 = reinterpret_cast<const float4*>(lq + t * DP + rg * RPL);
+        const float4* k4 = reinterpret_cast<const float4*>(lk + t * DP + rg * RPL);
+        float acc = 0.f, nq = 0.f;
+#pragma unroll
+        for (int i = 0; i < RPL; i += 4) {
+          const float4 qq = q4[i / 4], kk = k4[i / 4];
+          const float qa[4] = {qq.x, qq.y, qq.z, qq.w}, ka[4] = {kk.x, kk.y, kk.z, kk.w};
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            S[i + u] = fmaf(ka[u], tv, decay * S[i + u]);
+            nn[i + u] = fmaf(take, ka[u], decay * nn[i + u]);
+            acc = fmaf(S[i + u], qa[u], acc);
+            nq = fmaf(nn[i + u], qa[u], nq);
+          }
+        }
+        acc += __shfl_xor(acc, 16, TI_WAVE);
+        acc += __shfl_xor(acc, 32, TI_WAVE);
+        nq += __shfl_xor(nq, 16, TI_WAVE);
+        nq += __shfl_xor(nq, 32, TI_WAVE);
+        const float denom = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
+        if (rg == 0 && active) o[(size_t)(row0 + t0 + t) * ov + h * dv + j] = acc / denom;
+      }
+    }
+    if (active) {
+#pragma unroll
+      for (int i = 0; i < RPL; ++i) {
+        const int r = rg * RPL + i;
+        if (r < dk) S_base[(size_t)r * dv + j] = S[i];
+      }
+    }
+  }
+  // n and m: every lane holds the same; one lane per quarter of the rows writes, after all have read
+  __syncthreads();
+  if (wave == 0 && c == 0) {
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+      const int r = rg * RPL + i;
+      if (r < dk) n_base[r] = nn[i];
+    }
+    if (rg == 0) *m_ptr = m;
+  }
+}
+
+// proj f32 [M, ld]: the projections of the step's rows; off_*: the columns where the heads' q [heads][dk],
+// k [heads][dk], v [heads][dv] and the gate pre-activations i, f [heads] start.  state f32: per slot
+// (slot_stride floats apart) [heads][dk dv + dk + 1] = S row-major [dk][dv], n, m.  entries int32 [R][4] =
+// (first row, tokens, -, state slot).  o f32 [M, heads dv].
+extern "C" int ti_mlstm_scan(const float* proj, int ld, int off_q, int off_k, int off_v, int off_i, int off_f,
+                             const float* bias_i, const float* bias_f, float* state, long slot_stride, const int* entries,
+                             int n_entries, float* o, int heads, int dk, int dv, float cap, float q_scale,
+                             hipStream_t stream) {
+  TI_REQUIRE(heads > 0 && heads <= 65535 && dk >= 1 && dk <= 256 && dv >= 1, "mlstm: heads %d, key size %d (up to 256), value size %d",
+             heads, dk, dv);
+  TI_REQUIRE(cap > 0.f, "mlstm: the gates' cap must be positive");
+  if (n_entries == 0) return 0;
+  const int rpl = dk <= 32 ? 8 : dk <= 64 ? 16 : dk <= 128 ? 32 : 64;
+  const int max_waves = rpl <= 16 ? 16 : rpl == 32 ? 8 : 4;
+  int waves = (dv + ML_COLS - 1) / ML_COLS;
+  if (waves > max_waves) waves = max_waves;
+  const size_t lds = ((size_t)ML_TB * (2 * rpl * ML_RG + dv) + 2 * ML_TB) * sizeof(float);
+  TI_REQUIRE(lds <= 64 * 1024, "mlstm: value size %d needs %zu bytes of LDS", dv, lds);
+  dim3 grid(n_entries, heads);
+#define ML_GO(R, T)                                                                                                   \
+  mlstm_scan_kernel<R, T><<<grid, waves * 64, lds, stream>>>(proj, ld, off_q, off_k, off_v, off_i, off_f, bias_i, bias_f, \
+                                                             state, slot_stride, entries, o, heads, dk, dv, cap, q_scale)
+  if (rpl == 8) ML_GO(8, 1024);
+  else if (rpl == 16) ML_GO(16, 1024);
+  else if (rpl == 32) ML_GO(32, 512);
+  else ML_GO(64, 256);
+#undef ML_GO
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// out[m, h, j] = o[m, h, j] / sqrt(mean_j o[m, h, :]^2 + eps) * w[h dv + j] * sigmoid(gate[m, h dv + j])
+// (gate: rows of `ld` floats, the head's pre-activations from column off_g on), in T.  A wavefront per (row, head).
+template <typename T>
+__global__ void __launch_bounds__(64)
+gated_head_norm_kernel(const float* __restrict__ o, const float* __restrict__ gate, int ld, int off_g,
+                       const float* __restrict__ w, T* __restrict__ out, int heads, int dv, float eps) {
+  const int m = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* src = o + ((size_t)m * heads + h) * dv;
+  float ss = 0.f;
+  for (int j = lane; j < dv; j += TI_WAVE) ss = fmaf(src[j], src[j], ss);
+  const float scale = 1.0f / sqrtf(group_sum<TI_WAVE>(ss) / (float)dv + eps);
+  const float* g = gate + (size_t)m * ld + off_g + h * dv;
+  T* dst = out + ((size_t)m * heads + h) * dv;
+  for (int j = lane; j < dv; j += TI_WAVE) {
+    const float sg = 1.0f / (1.0f + expf(-g[j]));
+    st<T>(dst + j, src[j] * scale * w[h * dv + j] * sg);
+  }
+}
+
+extern "C" int ti_gated_head_norm(int out_dtype, const float* o, const float* gate, int ld, int off_g, const float* w,
+                                  void* out, int M, int heads, int dv, float eps, hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && heads > 0 && heads <= 65535 && dv > 0, "gated_head_norm: bad sizes M=%d heads=%d dv=%d", M, heads, dv);
+  if (M == 0) return 0;
+  dim3 grid(M, heads);
+  if (out_dtype == TI_F32)
+    gated_head_norm_kernel<float><<<grid, 64, 0, stream>>>(o, gate, ld, off_g, w, (float*)out, heads, dv, eps);
+  else if (out_dtype == TI_BF16)
+    gated_head_norm_kernel<bf16_t><<<grid, 64, 0, stream>>>(o, gate, ld, off_g, w, (bf16_t*)out, heads, dv, eps);
+  else
+    TI_REQUIRE(false, "gated_head_norm: unknown dtype %d", out_dtype);
+  TI_LAUNCH_CHECK();
+  return 0;
+}

@@ -92,6 +92,39 @@ int ti_attention_rows(int dtype, const void* q, const void* pool, const int* tab
                       const int* slot, void* out, int M, int n_head, int n_kv, int hd, int page_size, float scale,
                       int window, hipStream_t stream);
 
+// the same for keys and values of different sizes (dk, dv up to 256, any value in that range) and soft-capped scores:
+// s = (q . k) scale, then softcap tanh(s / softcap) if softcap > 0.  A page is K [n_kv][P][dk] | V [n_kv][dv][P].
+int ti_attention_capped_rows(int dtype, const void* q, const void* pool, const int* table, int table_stride,
+                             const int* pos, const int* slot, void* out, int M, int n_head, int n_kv, int dk, int dv,
+                             int page_size, float scale, float softcap, int window, hipStream_t stream);
+
+// ---- libti_pointwise: element-wise kernels of layers beyond the pre-norm transformer block
+// x[m, 2i] += sin(pos[m] inv_freq[i]), x[m, 2i + 1] += cos(pos[m] inv_freq[i])
+int ti_add_sinusoid(float* x, const int* pos, const float* inv_freq, int M, int H, hipStream_t stream);
+// x[m, :] += v
+int ti_add_row(float* x, const float* v, int M, int H, hipStream_t stream);
+// out = xIELU(z) with act = (p, q): z > 0: softplus(p) z^2 + z/2; else (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2
+int ti_xielu(int out_dtype, const float* z, const float* act, void* out, long n, hipStream_t stream);
+// x[m, c] += a[m, c] sa[c] + b[m, c] sb[c]  (b may be null; a scale that is null is 1)
+int ti_scaled_add(float* x, const float* a, const float* sa, const float* b, const float* sb, int M, int H,
+                  hipStream_t stream);
+// qkv f32 [M, n_head dk + n_kv dk + n_kv dv]: q times 1 + coef ln(floor((pos + 1) / every) + 1) to q_out, k and v into
+// the pages (layout as ti_attention_capped_rows reads it)
+int ti_qkv_split_write(int dtype, const float* qkv, const int* pos, const int* slot, const int* table, int table_stride,
+                       void* pool, void* q_out, int M, int n_head, int n_kv, int dk, int dv, int page_size, float coef,
+                       int every, hipStream_t stream);
+
+// ---- libti_recurrent: the mLSTM cell as a scan over each request's tokens of the step
+// proj f32 [M, ld] holds, from the columns off_* on, the heads' q and k [heads][dk], v [heads][dv] and the gates'
+// pre-activations i, f [heads]; state f32, slot_stride floats per slot: [heads][dk dv + dk + 1] (S [dk][dv], n, m);
+// entries int32 [n_entries][4] = (first row, tokens, -, state slot); o f32 [M, heads dv] (not yet normed)
+int ti_mlstm_scan(const float* proj, int ld, int off_q, int off_k, int off_v, int off_i, int off_f, const float* bias_i,
+                  const float* bias_f, float* state, long slot_stride, const int* entries, int n_entries, float* o,
+                  int heads, int dk, int dv, float cap, float q_scale, hipStream_t stream);
+// out = o / rms(o per head) * w * sigmoid(gate), gate in rows of ld floats from column off_g on
+int ti_gated_head_norm(int out_dtype, const float* o, const float* gate, int ld, int off_g, const float* w, void* out,
+                       int M, int heads, int dv, float eps, hipStream_t stream);
+
 // ---- libti_attention_bf16: the same on the matrix cores (head sizes 32, 64, 128; pages of 16 n rows)
 // rows of single tokens; n_splits > 1 needs part_o f32 [n_rows, n_head, n_splits, hd] and part_ml f32
 // [n_rows, n_head, n_splits, 2]

@@ -84,6 +84,7 @@ Json cache_need_json(const CacheNeed& n) {
     j.set("kind", "paged_kv");
     j.set("kv_heads", n.kv_heads);
     j.set("head_dim", n.head_dim);
+    if (n.value_dim() != n.head_dim) j.set("v_dim", n.v_dim);
     j.set("window", n.window > 0 ? Json(n.window) : Json());
   } else if (n.kind == CacheNeed::PagedRows) {
     j.set("kind", "paged_rows");
@@ -114,6 +115,7 @@ CacheNeed cache_need_from(const Json& c) {
     n.kind = CacheNeed::PagedKV;
     n.kv_heads = (int)c.at("kv_heads").as_int();
     n.head_dim = (int)c.at("head_dim").as_int();
+    n.v_dim = c.has("v_dim") ? (int)c.at("v_dim").as_int() : 0;
     n.window = c.has("window") ? (int)c.at("window").as_int() : 0;
   }
   return n;

@@ -550,7 +550,7 @@ Engine::Engine(std::shared_ptr<Model> model_, const EngineOptions& o)
   for (const auto& g : model->cache_groups) {
     size_t per_layer;
     if (g.first.kind == CacheNeed::PagedKV) {
-      per_layer = (size_t)num_pages * 2 * g.first.kv_heads * page_size * g.first.head_dim * dtype_size(act_dtype);
+      per_layer = (size_t)num_pages * g.first.kv_heads * page_size * (g.first.head_dim + g.first.value_dim()) * dtype_size(act_dtype);
     } else if (g.first.kind == CacheNeed::PagedRows) {
       if (g.first.row_shape.empty() || g.first.row_shape.size() > 2)
         throw EngineError("a paged cache of rows needs a row shape of one or two dimensions");
@@ -615,6 +615,10 @@ Tensor Engine::kv_pool(int group, int layer) const {
     if (shape.size() == 4) t = Tensor(t.data, t.dtype, {shape[0], shape[1], shape[2], shape[3]});
     return t;
   }
+  // values of another size than the keys: a page is K [kv heads][P][head_dim] | V [kv heads][v_dim][P]
+  if (g.first.value_dim() != g.first.head_dim)
+    return Tensor((char*)impl_->storage[group].data() + (size_t)layer * impl_->layer_bytes[group], act_dtype,
+                  {num_pages, (int64_t)g.first.kv_heads, (int64_t)page_size, (int64_t)(g.first.head_dim + g.first.value_dim())});
   return Tensor((char*)impl_->storage[group].data() + (size_t)layer * impl_->layer_bytes[group], act_dtype,
                 {num_pages, 2 * (int64_t)g.first.kv_heads, (int64_t)page_size, (int64_t)g.first.head_dim});
 }

@@ -35,7 +35,7 @@ namespace {
 struct Args {
   std::string model, dtype, out;
   long max_tokens = 0, num_pages = 0;
-  int page_size = 16, max_requests = 8, max_seq = 0;
+  int page_size = 16, max_requests = 4, max_seq = 0;
   bool random_weights = false;
   unsigned long long seed = 0;
   std::vector<std::string> plugins;

@@ -160,12 +160,15 @@ using SpecBuilder = std::function<ModelSpec(const Json& config)>;
 // filled in (what a model folder's config.json says after a round trip).  Optional.
 using ConfigReader = std::function<Json(const Json& config)>;
 void register_architecture(const std::vector<std::string>& names, SpecBuilder builder, ConfigReader typed = nullptr);
+// the Miterax decoder (config/miterax.cpp): its config.json read and validated, and its model as data
+Json miterax_typed_config(const Json& config);
+ModelSpec miterax_spec(const Json& config);
 // {"architecture": the registered name that matched, "config": the typed configuration (the input itself if
 // the architecture registered no reader)}; ConfigError as spec_from_config
 Json typed_config(const Json& config);
 std::vector<std::string> registered_architectures();
 bool architecture_registered(const Json& config);
-ModelSpec spec_from_config(const Json& config);   // by architectures[0], else model_type; ConfigError lists what is registered
+ModelSpec spec_from_config(const Json& config);   // by architectures[0], else model_type or architecture; ConfigError lists what is registered
 
 // ------------------------------------------------------------------------------------ tensors
 enum class DType : int { F32 = 0, BF16 = 1, I32 = 2, F16 = 3, F64 = 4, I64 = 5 };   // the kernels serve 0 and 1
@@ -241,6 +244,9 @@ struct CacheNeed {
   // (a mixer with another kind of memory than keys and values).  State: a fixed size per request.
   enum Kind { PagedKV, State, PagedRows } kind = PagedKV;
   int kv_heads = 0, head_dim = 0, window = 0;    // PagedKV; window (PagedRows too) 0: every token is kept
+  int v_dim = 0;                                 // PagedKV: the size of a value where it is not head_dim (0: it is).  A page
+                                                 // is then K [kv heads][P][head_dim] | V [kv heads][v_dim][P]
+  int value_dim() const { return v_dim > 0 ? v_dim : head_dim; }
   std::vector<int64_t> state_shape;              // State: float32 per request and layer, zeroed at admission
   std::vector<int64_t> row_shape;                // PagedRows: one or two dimensions, in the compute dtype ...
   bool rows_f32 = false;                         // ... or in float32
@@ -309,6 +315,29 @@ class Ops {
                                   const float* q_w, const float* k_w, float eps, const Rotation& rot, const Tensor& pool,
                                   bool write_kv, const Tensor& out, int heads, int kv_heads, int head_dim, float scale,
                                   int window);
+  // ---- layers beyond the pre-norm transformer block
+  // x[m, 2i] += sin(pos[m] inv_freq[i]), x[m, 2i + 1] += cos(the same)
+  void add_sinusoid(const Tensor& x, const int* positions, const Tensor& inv_freq);
+  void add_row(const Tensor& x, const Tensor& v);                                   // x[m, :] += v
+  // out = xIELU(z; act = (p, q)): z f32, out in the compute dtype
+  void xielu(const Tensor& z, const Tensor& act, const Tensor& out);
+  // x += a * sa + b * sb per channel (b / sb may be undefined: one branch)
+  void scaled_add(const Tensor& x, const Tensor& a, const Tensor& sa, const Tensor& b, const Tensor& sb);
+  // A fused q/k/v projection with keys of size dk and values of size dv: q times its temperature
+  // 1 + coef ln(floor((pos + 1) / every) + 1) to q_out, k and v into the pages (K [kv][P][dk] | V [kv][dv][P])
+  void qkv_split_write(const Tensor& qkv, const int* positions, const int* slots, const CacheView& view, const Tensor& pool,
+                       const Tensor& q_out, int heads, int kv_heads, int dk, int dv, float temp_coef, int temp_every);
+  // causal attention of every row over such pages, scores soft-capped: softcap tanh(s / softcap) (softcap 0: none)
+  void attention_capped(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
+                        const Tensor& out, int heads, int kv_heads, int dk, int dv, float scale, float softcap, int window);
+  // The mLSTM cell over each entry's tokens, from and into its state slot.  proj f32 [M, ld] with the heads' q, k, v and
+  // gate pre-activations from the given columns on; state f32 [slots][heads][dk dv + dk + 1]; o f32 [M, heads dv]
+  struct MlstmColumns { int q = 0, k = 0, v = 0, i = 0, f = 0; };
+  void mlstm_scan(const Tensor& proj, const MlstmColumns& cols, const Tensor& bias_i, const Tensor& bias_f, const Tensor& state,
+                  const int* entry_meta, int n_entries, const Tensor& o, int heads, int dk, int dv, float cap, float q_scale);
+  // out = o / rms(o per head) * w * sigmoid(gate columns of proj), in the compute dtype
+  void gated_head_norm(const Tensor& o, const Tensor& proj, int gate_col, const Tensor& w, float eps, const Tensor& out,
+                       int heads, int dv);
   void argmax(const Tensor& logits, int* out);
   void sample(const Tensor& logits, const float* temperature, const int* top_k, const float* top_p, const float* uniform,
               int* out);
@@ -528,12 +557,19 @@ class NormPart : public Part { public: using Part::Part; const char* family() co
   virtual bool can_be_lazy() const { return false; } };
 class PositionPart : public Part { public: using Part::Part; const char* family() const override { return "pos"; }
   virtual bool fused(Ops::Rotation& rot) const { return false; }    // arguments for the fused q/k kernels
+  virtual bool additive() const { return false; }                   // an encoding added to the residual behind the embedding ...
+  virtual void add(StepContext& ctx, const Tensor& x) {}            // ... x f32 [M, H] += its vectors at ctx.positions
   virtual void apply(StepContext& ctx, const Tensor& q, const Tensor& k) = 0; };   // f32 [M, heads, hd] views; k may be undefined
 class MixerPart : public Part { public: using Part::Part; const char* family() const override { return "mixer"; }
   virtual void forward(StepContext& ctx, const Rows& h, const Tensor& x) = 0;
+  // y f32 [M, H] = the part's output, nothing added: for arrangements that scale or combine outputs before the sum
+  virtual bool can_store() const { return false; }
+  virtual void forward_store(StepContext& ctx, const Rows& h, const Tensor& y);
   virtual bool takes_lazy_norm() const { return false; } };        // h goes into exactly one Ops::linear
 class FeedForwardPart : public Part { public: using Part::Part; const char* family() const override { return "ffn"; }
   virtual void forward(StepContext& ctx, const Rows& h, const Tensor& x) = 0;
+  virtual bool can_store() const { return false; }
+  virtual void forward_store(StepContext& ctx, const Rows& h, const Tensor& y);
   virtual bool takes_lazy_norm() const { return false; } };
 class BlockPart : public Part { public: using Part::Part; const char* family() const override { return "block"; }
   virtual void forward(StepContext& ctx, const Tensor& x) = 0; };

@@ -25,8 +25,12 @@ Model::Model(const ModelSpec& s) : spec(s) {
       const PartSpec* ps = nullptr;
       for (const auto& kv : ls.parts)
         if (kv.first == slot.first) ps = &kv.second;
+      // a slot whose family ends in '?' may stay empty
+      const bool optional = !slot.second.empty() && slot.second.back() == '?';
+      if (!ps && optional) continue;
       if (!ps) throw ConfigError("layer '" + ls.prefix + "': block '" + ls.block.kind + "' needs a '" + slot.first + "' part");
-      built.emplace_back(slot.first, build_part(slot.second, *ps, join(ls.prefix, ps->name)));
+      const std::string family = optional ? slot.second.substr(0, slot.second.size() - 1) : slot.second;
+      built.emplace_back(slot.first, build_part(family, *ps, join(ls.prefix, ps->name)));
     }
     blocks.push_back(std::dynamic_pointer_cast<BlockPart>(build_part("block", ls.block, ls.prefix, built)));
   }

@@ -854,6 +854,130 @@ void Ops::attention(const AttentionWork& work, Workspace& ws, const CacheView& v
     attention_rows(q, pool, view, work.positions, work.slots, out, heads, kv_heads, head_dim, scale, window);
 }
 
+// ------------------------------------------------- layers beyond the pre-norm transformer block
+void Ops::add_sinusoid(const Tensor& x, const int* positions, const Tensor& inv_freq) {
+  TIMED("add_sinusoid " + dims(x));
+  require(x.ndim == 2 && x.dtype == DType::F32 && x.contiguous(), "add_sinusoid: x must be contiguous float32 [M, H]");
+  require(inv_freq.dtype == DType::F32 && inv_freq.numel() == (x.shape[1] + 1) / 2,
+          "add_sinusoid: inv_freq must be float32 [ceil(H / 2)]");
+  int rc = KERNEL("pointwise", ti_add_sinusoid)((float*)x.data, positions, (const float*)inv_freq.data, (int)x.shape[0],
+                                                (int)x.shape[1], (hipStream_t)launch_stream());
+  check("pointwise", rc, "add_sinusoid");
+}
+
+void Ops::add_row(const Tensor& x, const Tensor& v) {
+  TIMED("add_row " + dims(x));
+  require(x.ndim == 2 && x.dtype == DType::F32 && x.contiguous() && v.dtype == DType::F32 && v.numel() == x.shape[1],
+          "add_row: x " + x.describe() + " and v " + v.describe() + " do not fit");
+  int rc = KERNEL("pointwise", ti_add_row)((float*)x.data, (const float*)v.data, (int)x.shape[0], (int)x.shape[1],
+                                           (hipStream_t)launch_stream());
+  check("pointwise", rc, "add_row");
+}
+
+void Ops::xielu(const Tensor& z, const Tensor& act, const Tensor& out) {
+  TIMED("xielu " + dims(z));
+  require(z.dtype == DType::F32 && z.contiguous() && out.contiguous() && out.numel() == z.numel() && act.dtype == DType::F32 &&
+              act.numel() == 2,
+          "xielu: z " + z.describe() + ", out " + out.describe() + " or act " + act.describe() + " do not fit");
+  int rc = KERNEL("pointwise", ti_xielu)(code(out.dtype, "xielu"), (const float*)z.data, (const float*)act.data, out.data,
+                                         (long)z.numel(), (hipStream_t)launch_stream());
+  check("pointwise", rc, "xielu");
+}
+
+void Ops::scaled_add(const Tensor& x, const Tensor& a, const Tensor& sa, const Tensor& b, const Tensor& sb) {
+  TIMED("scaled_add " + dims(x));
+  const int64_t H = x.ndim == 2 ? x.shape[1] : 0;
+  auto fits = [&](const Tensor& t) { return t.dtype == DType::F32 && t.contiguous() && t.numel() == x.numel(); };
+  auto scale_fits = [&](const Tensor& t) { return !t.defined() || (t.dtype == DType::F32 && t.numel() == H); };
+  require(x.ndim == 2 && fits(x) && fits(a) && (!b.defined() || fits(b)) && scale_fits(sa) && scale_fits(sb),
+          "scaled_add: the operands do not fit x " + x.describe());
+  int rc = KERNEL("pointwise", ti_scaled_add)((float*)x.data, (const float*)a.data, (const float*)sa.data, (const float*)b.data,
+                                              b.defined() ? (const float*)sb.data : nullptr, (int)x.shape[0], (int)H,
+                                              (hipStream_t)launch_stream());
+  check("pointwise", rc, "scaled_add");
+}
+
+// a pool of one cache layer whose keys and values differ in size is [pages][kv heads][P][dk + dv]
+static void check_split_pool(const char* what, const Tensor& pool, int kv_heads, int dk, int dv, DType dt) {
+  require(pool.ndim == 4 && pool.dtype == dt && pool.contiguous() &&
+              pool.shape[1] * pool.shape[3] == (int64_t)kv_heads * (dk + dv),
+          std::string(what) + ": pool " + pool.describe() + " does not hold " + std::to_string(kv_heads) + " kv heads of " +
+              std::to_string(dk) + " + " + std::to_string(dv) + " in " + dtype_name(dt));
+}
+
+void Ops::qkv_split_write(const Tensor& qkv, const int* positions, const int* slots, const CacheView& view, const Tensor& pool,
+                          const Tensor& q_out, int heads, int kv_heads, int dk, int dv, float temp_coef, int temp_every) {
+  TIMED("qkv_split_write " + dims(qkv));
+  const int64_t M = qkv.shape[0];
+  const int64_t width = (int64_t)heads * dk + (int64_t)kv_heads * (dk + dv);
+  require(qkv.ndim == 2 && qkv.shape[1] == width && qkv.dtype == DType::F32 && qkv.contiguous(),
+          "qkv_split_write: qkv " + qkv.describe() + " does not fit [M, " + std::to_string(width) + "] float32");
+  require(q_out.ndim == 2 && q_out.shape[0] == M && q_out.shape[1] == (int64_t)heads * dk && q_out.contiguous(),
+          "qkv_split_write: q_out has the wrong shape");
+  check_split_pool("qkv_split_write", pool, kv_heads, dk, dv, q_out.dtype);
+  int rc = KERNEL("pointwise", ti_qkv_split_write)(code(q_out.dtype, "qkv_split_write"), (const float*)qkv.data, positions, slots,
+                                                   view.table, view.table_width, pool.data, q_out.data, (int)M, heads, kv_heads,
+                                                   dk, dv, (int)pool.shape[2], temp_coef, temp_every,
+                                                   (hipStream_t)launch_stream());
+  check("pointwise", rc, "qkv_split_write");
+}
+
+void Ops::attention_capped(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
+                           const Tensor& out, int heads, int kv_heads, int dk, int dv, float scale, float softcap, int window) {
+  TIMED("attention_capped " + dims(q));
+  const int64_t M = q.shape[0];
+  require(q.ndim == 2 && q.shape[1] == (int64_t)heads * dk && out.ndim == 2 && out.shape[0] == M &&
+              out.shape[1] == (int64_t)heads * dv && q.dtype == pool.dtype && out.dtype == q.dtype && q.contiguous() &&
+              out.contiguous(),
+          "attention_capped: q/out/pool shapes or dtypes do not fit");
+  check_split_pool("attention_capped", pool, kv_heads, dk, dv, q.dtype);
+  took("[generic]");
+  int rc = KERNEL("attention_generic", ti_attention_capped_rows)(
+      code(q.dtype, "attention_capped"), q.data, pool.data, view.table, view.table_width, positions, slots, out.data, (int)M,
+      heads, kv_heads, dk, dv, (int)pool.shape[2], scale, softcap, window, (hipStream_t)launch_stream());
+  check("attention_generic", rc, "attention_capped");
+}
+
+void Ops::mlstm_scan(const Tensor& proj, const MlstmColumns& cols, const Tensor& bias_i, const Tensor& bias_f, const Tensor& state,
+                     const int* entry_meta, int n_entries, const Tensor& o, int heads, int dk, int dv, float cap, float q_scale) {
+  TIMED("mlstm_scan " + dims(proj) + " entries=" + std::to_string(n_entries));
+  const int64_t per_head = (int64_t)dk * dv + dk + 1;
+  require(proj.ndim == 2 && proj.dtype == DType::F32 && proj.contiguous(), "mlstm_scan: proj must be contiguous float32 [M, N]");
+  const int64_t N = proj.shape[1];
+  require(cols.q >= 0 && cols.q + (int64_t)heads * dk <= N && cols.k >= 0 && cols.k + (int64_t)heads * dk <= N && cols.v >= 0 &&
+              cols.v + (int64_t)heads * dv <= N && cols.i >= 0 && cols.i + heads <= N && cols.f >= 0 && cols.f + heads <= N,
+          "mlstm_scan: the columns do not lie inside proj " + proj.describe());
+  require(state.dtype == DType::F32 && state.contiguous() && state.ndim >= 2 && state.numel() == state.shape[0] * heads * per_head,
+          "mlstm_scan: state " + state.describe() + " does not fit [slots, " + std::to_string(heads) + ", " +
+              std::to_string(per_head) + "]");
+  require(bias_i.dtype == DType::F32 && bias_i.numel() == heads && bias_f.dtype == DType::F32 && bias_f.numel() == heads,
+          "mlstm_scan: the gates' biases must be float32 [heads]");
+  require(o.dtype == DType::F32 && o.contiguous() && o.ndim == 2 && o.shape[0] == proj.shape[0] && o.shape[1] == (int64_t)heads * dv,
+          "mlstm_scan: o " + o.describe() + " does not fit");
+  require(entry_meta != nullptr || n_entries == 0, "mlstm_scan: no entry records");
+  int rc = KERNEL("recurrent", ti_mlstm_scan)((const float*)proj.data, (int)N, cols.q, cols.k, cols.v, cols.i, cols.f,
+                                              (const float*)bias_i.data, (const float*)bias_f.data, (float*)state.data,
+                                              (long)(heads * per_head), entry_meta, n_entries, (float*)o.data, heads, dk, dv, cap,
+                                              q_scale, (hipStream_t)launch_stream());
+  check("recurrent", rc, "mlstm_scan");
+}
+
+void Ops::gated_head_norm(const Tensor& o, const Tensor& proj, int gate_col, const Tensor& w, float eps, const Tensor& out,
+                          int heads, int dv) {
+  TIMED("gated_head_norm " + dims(o));
+  const int64_t M = o.shape[0], W = (int64_t)heads * dv;
+  require(o.ndim == 2 && o.dtype == DType::F32 && o.contiguous() && o.shape[1] == W && out.ndim == 2 && out.shape[0] == M &&
+              out.shape[1] == W && out.contiguous() && w.dtype == DType::F32 && w.numel() == W,
+          "gated_head_norm: o " + o.describe() + ", out " + out.describe() + " or w " + w.describe() + " do not fit");
+  require(proj.ndim == 2 && proj.dtype == DType::F32 && proj.contiguous() && proj.shape[0] == M && gate_col >= 0 &&
+              gate_col + W <= proj.shape[1],
+          "gated_head_norm: the gate's columns do not lie inside proj " + proj.describe());
+  int rc = KERNEL("recurrent", ti_gated_head_norm)(code(out.dtype, "gated_head_norm"), (const float*)o.data,
+                                                   (const float*)proj.data, (int)proj.shape[1], gate_col, (const float*)w.data,
+                                                   out.data, (int)M, heads, dv, eps, (hipStream_t)launch_stream());
+  check("recurrent", rc, "gated_head_norm");
+}
+
 // ----------------------------------------------------------------------------------- sampling
 void Ops::argmax(const Tensor& logits, int* out) {
   TIMED("argmax " + dims(logits));

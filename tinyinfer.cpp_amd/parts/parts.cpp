@@ -17,6 +17,17 @@
 //   head      "linear"    logits = h E_out^T with E_out the embedding itself or a matrix of its own
 //                         (/root/reference/src/cuda/lm_head.cu:5-10; the reference is always tied, src/model.h:42)
 //
+//
+// Parts no layer of the reference has (their formulas stand at each class):
+//   pos       "sinusoidal"  a vector of sines and cosines of the position added to the residual behind the embedding
+//   norm      "rmsnorm" with `scalar`: one learned number as the gain of every channel
+//   mixer     "attention" with `v_head_dim`, `softcap`, `q_temp`: keys and values of different sizes, tanh-capped
+//                           scores, a query factor that grows with the logarithm of the position
+//   mixer     "mlstm"       the mLSTM cell: a matrix memory per head, kept as per-request state
+//   ffn       "dense"       down(act(up h)) with the xIELU activation
+//   block     "parallel"    x += s1 * mixer(norm(x)) + s2 * ffn(norm(x)) with learned per-channel scales
+//   block     "add_vector"  x += a row of a learned table (what a looped run of layers adds before each pass)
+//
 // A part gets every size and constant as a parameter and never looks at the model it sits in.
 #include <algorithm>
 #include <cmath>
@@ -71,7 +82,21 @@ double param_float(const Json& p, const char* key) {
   if (!v || !v->is_number()) throw ConfigError(std::string("part parameter '") + key + "' is missing or not a number");
   return v->as_double();
 }
+// a tensor's name in the checkpoint: the parameter `key` gives it in full, else prefix + "." + fallback
+std::string tensor_name(const Json& p, const char* key, const std::string& prefix, const char* fallback) {
+  const Json* v = p.find(key);
+  if (v && v->type() == Json::String) return v->as_string();
+  if (prefix.empty()) return fallback;
+  return prefix + "." + fallback;
+}
 }  // namespace
+
+void MixerPart::forward_store(StepContext&, const Rows&, const Tensor&) {
+  throw EngineError(std::string("the mixer '") + kind_name() + "' cannot write its output apart from the residual");
+}
+void FeedForwardPart::forward_store(StepContext&, const Rows&, const Tensor&) {
+  throw EngineError(std::string("the feed-forward '") + kind_name() + "' cannot write its output apart from the residual");
+}
 
 void register_part(const std::string& family, const std::string& kind, PartFactory factory,
                    std::vector<std::pair<std::string, std::string>> slots) {
@@ -134,20 +159,41 @@ std::shared_ptr<Part> build_part(const std::string& family, const PartSpec& spec
 // ------------------------------------------------------------------------------- built-in parts
 namespace {
 
+// `tensor`: the table's name in the checkpoint (default: prefix + ".weight").  `pos`: an additive position
+// encoding (a part of family "pos" with additive() true), added to every row behind the lookup.
 class Embedding final : public EmbeddingPart {
  public:
-  Embedding(const std::string& prefix, int64_t vocab, int64_t dim) : EmbeddingPart(prefix), vocab(vocab), dim(dim) {}
+  Embedding(const std::string& prefix, const Json& p, const PartChildren& children)
+      : EmbeddingPart(prefix), vocab(param_int(p, "vocab")), dim(param_int(p, "dim")), name(tensor_name(p, "tensor", prefix, "weight")) {
+    for (const auto& c : children)
+      if (c.first == "pos") pos = std::dynamic_pointer_cast<PositionPart>(c.second);
+    if (!pos && p.has("pos")) pos = std::dynamic_pointer_cast<PositionPart>(build_part("pos", PartSpec::from_json(p.at("pos")), prefix));
+    if (pos && !pos->additive()) throw ConfigError("embedding: the position encoding '" + std::string(pos->kind_name()) + "' is not additive");
+  }
   const char* kind_name() const override { return "table"; }
   std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
     TensorNeed n;
     n.shape = {vocab, dim};
-    return {{join(prefix, "weight"), n}};
+    return {{name, n}};
   }
-  void load(WeightSource& src) override { weight = src.fetch(join(prefix, "weight"), tensors()[0].second); }
-  void forward(StepContext& ctx, const Tensor& x) override { ctx.ops.embed(weight, ctx.tokens, ctx.M, x, ctx.fed_tokens, ctx.n_fed_tokens); }
+  std::vector<std::shared_ptr<Part>> children() const override {
+    if (pos) return {pos};
+    return {};
+  }
+  std::vector<std::string> child_slots() const override {
+    if (pos) return {"pos"};
+    return {};
+  }
+  void load(WeightSource& src) override { weight = src.fetch(name, tensors()[0].second); }
+  void forward(StepContext& ctx, const Tensor& x) override {
+    ctx.ops.embed(weight, ctx.tokens, ctx.M, x, ctx.fed_tokens, ctx.n_fed_tokens);
+    if (pos) pos->add(ctx, x);
+  }
   bool reads_through_ops() const override { return true; }
   std::vector<std::pair<std::string, Tensor>> held() const override { return {{"weight", weight}}; }
   int64_t vocab, dim;
+  std::string name;
+  std::shared_ptr<PositionPart> pos;
   Tensor weight;
 };
 
@@ -155,20 +201,20 @@ class Embedding final : public EmbeddingPart {
 // holds one and `tied_to` otherwise.
 class LMHead final : public HeadPart {
  public:
-  LMHead(const std::string& prefix, int64_t vocab, int64_t dim, int tied, std::string tied_to)
-      : HeadPart(prefix), vocab(vocab), dim(dim), tied(tied), tied_to(std::move(tied_to)) {}
+  LMHead(const std::string& prefix, int64_t vocab, int64_t dim, int tied, std::string tied_to, std::string own_name)
+      : HeadPart(prefix), vocab(vocab), dim(dim), tied(tied), tied_to(std::move(tied_to)), own_name(std::move(own_name)) {}
   const char* kind_name() const override { return "linear"; }
   std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
     TensorNeed must, may;
     must.shape = may.shape = {vocab, dim};
     may.optional = true;
-    const std::string own = join(prefix, "weight");
+    const std::string& own = own_name;
     if (tied == 0) return {{own, must}};
     // a checkpoint that still carries the duplicate is accepted
     return {{tied_to, must}, {own, may}};
   }
   void load(WeightSource& src) override {
-    const std::string own = join(prefix, "weight");
+    const std::string& own = own_name;
     TensorNeed n;
     n.shape = {vocab, dim};
     if (tied == 0 || (tied < 0 && src.has(own))) weight = src.fetch(own, n);
@@ -184,25 +230,38 @@ class LMHead final : public HeadPart {
   std::vector<std::pair<std::string, Tensor>> held() const override { return {{"weight", weight}}; }
   int64_t vocab, dim;
   int tied;
-  std::string tied_to;
+  std::string tied_to, own_name;
   Tensor weight;
 };
 
+// `scalar`: the checkpoint holds one number, the gain of every channel (y = x / rms(x) * g); it is spread
+// over a vector when the weights load, so every kernel that takes a norm's weight serves it.  `tensor`:
+// the weight's name in the checkpoint (default: prefix + ".weight").
 class RMSNorm final : public NormPart {
  public:
-  RMSNorm(const std::string& prefix, int64_t dim, double eps) : NormPart(prefix), dim(dim), eps((float)eps) {}
+  RMSNorm(const std::string& prefix, int64_t dim, double eps, bool scalar = false, std::string name_ = "")
+      : NormPart(prefix), dim(dim), eps((float)eps), scalar(scalar), name(name_.empty() ? join(prefix, "weight") : std::move(name_)) {}
   const char* kind_name() const override { return "rmsnorm"; }
   bool can_be_lazy() const override { return true; }
   bool reads_through_ops() const override { return true; }
   std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
     TensorNeed n;
-    n.shape = {dim};
+    if (!scalar) n.shape = {dim};
     n.role = TensorNeed::Vector;
     n.a = 1.0;
     n.b = 0.1;
-    return {{join(prefix, "weight"), n}};
+    return {{name, n}};
   }
-  void load(WeightSource& src) override { weight = src.fetch(join(prefix, "weight"), tensors()[0].second); }
+  void load(WeightSource& src) override {
+    if (!scalar) {
+      weight = src.fetch(name, tensors()[0].second);
+      return;
+    }
+    const Tensor one = src.fetch(name, tensors()[0].second);
+    weight = src.alloc(DType::F32, {dim});
+    spread(one, weight, src.to_host);
+  }
+  static void spread(const Tensor& one, const Tensor& all, bool on_host);     // all[:] = one[0]
   // x: f32 [M, dim].  With `rows` only those rows of x are read, in that order.  `lazy`: the
   // consumer feeds the result to one product and nothing else, so where a kernel can take the
   // norm in, the rows come back not yet computed.
@@ -223,7 +282,45 @@ class RMSNorm final : public NormPart {
   std::vector<std::pair<std::string, Tensor>> held() const override { return {{"weight", weight}}; }
   int64_t dim;
   float eps;
+  bool scalar;
+  std::string name;
   Tensor weight;
+};
+
+// An additive position encoding: entry 2i of a position's vector is sin(p * base^(-2i / dim)), entry 2i + 1 the
+// cosine of the same angle.  The frequencies are built on the host in double precision and rounded to 32-bit;
+// the angle and its sine and cosine are 32-bit on the device.
+class Sinusoidal final : public PositionPart {
+ public:
+  Sinusoidal(const std::string& prefix, int64_t dim, double base) : PositionPart(prefix), dim(dim), base(base) {
+    if (dim <= 0 || !(base > 0.0)) throw ConfigError("sinusoidal positions: dim and base must be positive");
+  }
+  const char* kind_name() const override { return "sinusoidal"; }
+  bool additive() const override { return true; }
+  bool reads_through_ops() const override { return true; }
+  void prepare(Ops&, int) override {
+    if (inv_freq.data()) return;
+    const int64_t half = (dim + 1) / 2;
+    std::vector<float> host((size_t)half);
+    for (int64_t i = 0; i < half; ++i) host[(size_t)i] = (float)std::pow(base, -2.0 * (double)i / (double)dim);
+    inv_freq = DeviceBuffer((size_t)half * 4);
+    upload(inv_freq.data(), host.data(), (size_t)half * 4);
+  }
+  void add(StepContext& ctx, const Tensor& x) override {
+    prepare(ctx.ops, 0);
+    ctx.ops.add_sinusoid(x, ctx.positions, Tensor(inv_freq.data(), DType::F32, {(dim + 1) / 2}));
+  }
+  void apply(StepContext&, const Tensor&, const Tensor&) override {
+    throw EngineError("sinusoidal positions are added to the residual; they do not rotate queries and keys");
+  }
+  std::vector<std::pair<std::string, Tensor>> held() const override {
+    if (!inv_freq.data()) return {};
+    return {{"inv_freq", Tensor(inv_freq.data(), DType::F32, {(dim + 1) / 2})}};
+  }
+  static void upload(void* dst, const void* src, size_t bytes);
+  int64_t dim;
+  double base;
+  DeviceBuffer inv_freq;
 };
 
 // The inverse frequencies are built once on the host in double precision and rounded to float.
@@ -369,11 +466,30 @@ class Attention final : public MixerPart {
     head_dim = (int)param_int(p, "head_dim");
     if (heads <= 0 || kv_heads <= 0 || heads % kv_heads)
       throw ConfigError("attention: heads " + std::to_string(heads) + " not a multiple of kv_heads " + std::to_string(kv_heads));
-    // every attention kernel's range (float32 and bfloat16 alike): refused when the part is built, not at its first step
-    if (head_dim < 16 || head_dim % 16 || head_dim > 256)
+    v_dim = p.has("v_head_dim") ? (int)param_int(p, "v_head_dim") : head_dim;
+    softcap = p.has("softcap") ? (float)param_float(p, "softcap") : 0.f;
+    if (p.has("q_temp")) {
+      const Json& qt = p.at("q_temp");
+      temp_coef = (float)param_float(qt, "coef");
+      temp_every = (int)param_int(qt, "every");
+      if (temp_every <= 0) throw ConfigError("attention: q_temp.every must be positive");
+    }
+    qk_norm = p.has("qk_norm") ? p.at("qk_norm").as_bool() : true;
+    // capped scores, a query temperature or values of another size than the keys: the kernels that serve these take
+    // any sizes up to 256 and neither a per-head norm nor a rotation
+    general = softcap > 0.f || temp_coef != 0.f || v_dim != head_dim || (p.has("general") && p.at("general").as_bool());
+    if (general) {
+      if (head_dim < 1 || head_dim > 256 || v_dim < 1 || v_dim > 256)
+        throw ConfigError("attention: key size " + std::to_string(head_dim) + " / value size " + std::to_string(v_dim) +
+                          " are not served (up to 256)");
+      if (qk_norm || p.has("pos") || (p.has("shares_kv") && p.at("shares_kv").as_bool()))
+        throw ConfigError("attention: capped scores, a query temperature or a separate value size go with neither a per-head norm, "
+                          "a rotation nor a shared cache");
+    } else if (head_dim < 16 || head_dim % 16 || head_dim > 256) {
+      // every other attention kernel's range (float32 and bfloat16 alike): refused when the part is built, not at its first step
       throw ConfigError("attention: head_dim " + std::to_string(head_dim) +
                         " is not served: the attention kernels take head sizes in steps of 16 up to 256");
-    qk_norm = p.has("qk_norm") ? p.at("qk_norm").as_bool() : true;
+    }
     eps = (float)(p.has("eps") ? p.at("eps").as_double() : 1e-6);
     window = p.has("window") ? (int)p.at("window").as_int() : 0;
     scale = p.has("scale") ? (float)p.at("scale").as_double() : (float)(1.0 / std::sqrt((double)head_dim));
@@ -383,8 +499,15 @@ class Attention final : public MixerPart {
     if (!pos && p.has("pos")) pos = std::dynamic_pointer_cast<PositionPart>(build_part("pos", PartSpec::from_json(p.at("pos")), prefix));
     nq = (int64_t)heads * head_dim;
     nk = shares_kv ? 0 : (int64_t)kv_heads * head_dim;
+    nv = shares_kv ? 0 : (int64_t)kv_heads * v_dim;
+    no = (int64_t)heads * v_dim;
+    n_q = tensor_name(p, "q", prefix, "q_proj.weight");
+    n_k = tensor_name(p, "k", prefix, "k_proj.weight");
+    n_v = tensor_name(p, "v", prefix, "v_proj.weight");
+    n_o = tensor_name(p, "o", prefix, "o_proj.weight");
   }
   const char* kind_name() const override { return "attention"; }
+  bool can_store() const override { return general; }
   bool takes_lazy_norm() const override { return true; }
   bool reads_through_ops() const override { return true; }
   std::vector<std::shared_ptr<Part>> children() const override {
@@ -397,19 +520,20 @@ class Attention final : public MixerPart {
   }
   std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
     std::vector<std::pair<std::string, TensorNeed>> t;
-    TensorNeed q, kv, o, nw;
+    TensorNeed q, kv, vv, o, nw;
     q.shape = {nq, hidden};
     kv.shape = {nk, hidden};
-    o.shape = {hidden, nq};
+    vv.shape = {nv, hidden};
+    o.shape = {hidden, no};
     nw.shape = {head_dim};
     nw.role = TensorNeed::Vector;
     nw.a = 1.0;
     nw.b = 0.1;
-    t.emplace_back(join(prefix, "q_proj.weight"), q);
-    t.emplace_back(join(prefix, "o_proj.weight"), o);
+    t.emplace_back(n_q, q);
+    t.emplace_back(n_o, o);
     if (!shares_kv) {
-      t.emplace_back(join(prefix, "k_proj.weight"), kv);
-      t.emplace_back(join(prefix, "v_proj.weight"), kv);
+      t.emplace_back(n_k, kv);
+      t.emplace_back(n_v, vv);
     }
     if (qk_norm) {
       t.emplace_back(join(prefix, "q_norm.weight"), nw);
@@ -420,14 +544,14 @@ class Attention final : public MixerPart {
   void load(WeightSource& src) override {
     // q, k and v go straight into the fused matrix (the reference builds its fused copy beside the
     // originals and keeps both: /root/reference/src/inference.cu:154-169)
-    w_qkv = src.alloc(src.matrix_dtype, {nq + 2 * nk, hidden});
-    src.fill(join(prefix, "q_proj.weight"), w_qkv.rows(0, nq));
+    w_qkv = src.alloc(src.matrix_dtype, {nq + nk + nv, hidden});
+    src.fill(n_q, w_qkv.rows(0, nq));
     if (!shares_kv) {
-      src.fill(join(prefix, "k_proj.weight"), w_qkv.rows(nq, nk));
-      src.fill(join(prefix, "v_proj.weight"), w_qkv.rows(nq + nk, nk));
+      src.fill(n_k, w_qkv.rows(nq, nk));
+      src.fill(n_v, w_qkv.rows(nq + nk, nv));
     }
-    w_o = src.alloc(src.matrix_dtype, {hidden, nq});
-    src.fill(join(prefix, "o_proj.weight"), w_o);
+    w_o = src.alloc(src.matrix_dtype, {hidden, no});
+    src.fill(n_o, w_o);
     if (qk_norm) {
       TensorNeed nw;
       nw.shape = {head_dim};
@@ -442,6 +566,7 @@ class Attention final : public MixerPart {
     n.kind = CacheNeed::PagedKV;
     n.kv_heads = kv_heads;
     n.head_dim = head_dim;
+    n.v_dim = v_dim != head_dim ? v_dim : 0;
     n.window = window;
     return n;
   }
@@ -519,7 +644,28 @@ class Attention final : public MixerPart {
     return w;
   }
 
+  // Capped scores, a query temperature, values of their own size: the projections in 32-bit, q times its temperature
+  // and k, v into the pages, attention with scores, cap and softmax in 32-bit, then the output projection.
+  void run_general(StepContext& ctx, const Rows& h, const Tensor& out, Ops::Epilogue epi) {
+    const int64_t M = h.t.shape[0];
+    Tensor qkv = ctx.buf("attn.qkv", DType::F32, {M, nq + nk + nv});
+    ctx.ops.linear(h, w_qkv, qkv, Ops::Store);
+    const auto bound = ctx.binding(this);
+    const Tensor pool = ctx.kv_pool(bound.first, bound.second);
+    const Ops::CacheView view = ctx.cache_view(bound.first);
+    Tensor q = ctx.buf("attn.q", ctx.act_dtype, {M, nq});
+    ctx.ops.qkv_split_write(qkv, ctx.positions, ctx.slots, view, pool, q, heads, kv_heads, head_dim, v_dim, temp_coef, temp_every);
+    Tensor a = ctx.buf("attn.out", ctx.act_dtype, {M, no});
+    ctx.ops.attention_capped(q, pool, view, ctx.positions, ctx.slots, a, heads, kv_heads, head_dim, v_dim, scale, softcap, window);
+    ctx.ops.linear(a, w_o, out, epi, epi == Ops::Add);
+  }
+  void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override {
+    if (!general) return MixerPart::forward_store(ctx, h, y);
+    run_general(ctx, h, y, Ops::Store);
+  }
+
   void forward(StepContext& ctx, const Rows& h, const Tensor& x) override {
+    if (general) return run_general(ctx, h, x, Ops::Add);
     const int64_t M = h.t.shape[0];
     const int64_t width = nq + 2 * nk;
     Tensor q = ctx.buf("attn.q", ctx.act_dtype, {M, nq});
@@ -578,10 +724,11 @@ class Attention final : public MixerPart {
   std::vector<std::pair<std::string, Tensor>> held() const override {
     return {{"w_qkv", w_qkv}, {"w_o", w_o}, {"q_norm_w", q_norm_w}, {"k_norm_w", k_norm_w}};
   }
-  int64_t hidden = 0, nq = 0, nk = 0;
-  int heads = 0, kv_heads = 0, head_dim = 0, window = 0;
-  bool qk_norm = true, shares_kv = false;
-  float eps = 1e-6f, scale = 1.f;
+  int64_t hidden = 0, nq = 0, nk = 0, nv = 0, no = 0;
+  int heads = 0, kv_heads = 0, head_dim = 0, v_dim = 0, window = 0, temp_every = 0;
+  bool qk_norm = true, shares_kv = false, general = false;
+  float eps = 1e-6f, scale = 1.f, softcap = 0.f, temp_coef = 0.f;
+  std::string n_q, n_k, n_v, n_o;
   std::shared_ptr<PositionPart> pos;
   Tensor w_qkv, w_o, q_norm_w, k_norm_w;
 };
@@ -620,21 +767,306 @@ class PreNormBlock final : public BlockPart {
   std::shared_ptr<FeedForwardPart> ffn;
 };
 
+// down(act(up h)) with act = xIELU and its two learned numbers (p, q) in the tensor `act`:
+//   z > 0: softplus(p) z^2 + z / 2;   z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2.
+// The first product leaves 32-bit sums, the activation is taken in 32-bit and rounded once to the compute dtype.
+// Tensor names: prefix + ".up", ".down", ".act" unless the parameters `up`, `down`, `act` give them in full.
+class DenseFFN final : public FeedForwardPart {
+ public:
+  DenseFFN(const std::string& prefix, const Json& p) : FeedForwardPart(prefix) {
+    hidden = param_int(p, "hidden");
+    intermediate = param_int(p, "intermediate");
+    const std::string act = p.has("activation") ? p.at("activation").as_string() : "xielu";
+    if (act != "xielu") throw ConfigError("dense feed-forward: activation '" + act + "' is not served (only 'xielu')");
+    if (hidden <= 0 || intermediate <= 0) throw ConfigError("dense feed-forward: sizes must be positive");
+    n_up = tensor_name(p, "up", prefix, "up");
+    n_down = tensor_name(p, "down", prefix, "down");
+    n_act = tensor_name(p, "act", prefix, "act");
+  }
+  const char* kind_name() const override { return "dense"; }
+  bool reads_through_ops() const override { return true; }
+  bool can_store() const override { return true; }
+  std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
+    TensorNeed up, down, act;
+    up.shape = {intermediate, hidden};
+    down.shape = {hidden, intermediate};
+    act.shape = {2};
+    act.role = TensorNeed::Vector;
+    act.a = 0.5;
+    act.b = 0.2;
+    return {{n_up, up}, {n_down, down}, {n_act, act}};
+  }
+  void load(WeightSource& src) override {
+    const auto t = tensors();
+    w_up = src.fetch(n_up, t[0].second);
+    w_down = src.fetch(n_down, t[1].second);
+    act = src.fetch(n_act, t[2].second);
+  }
+  void run(StepContext& ctx, const Rows& h, const Tensor& out, Ops::Epilogue epi) {
+    const int64_t M = h.t.shape[0];
+    Tensor z = ctx.buf("ffn.z", DType::F32, {M, intermediate});
+    ctx.ops.linear(h, w_up, z, Ops::Store);
+    Tensor y = ctx.buf("ffn.y", ctx.act_dtype, {M, intermediate});
+    ctx.ops.xielu(z, act, y);
+    ctx.ops.linear(y, w_down, out, epi, epi == Ops::Add);
+  }
+  void forward(StepContext& ctx, const Rows& h, const Tensor& x) override { run(ctx, h, x, Ops::Add); }
+  void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override { run(ctx, h, y, Ops::Store); }
+  std::vector<std::pair<std::string, Tensor>> held() const override { return {{"w_up", w_up}, {"w_down", w_down}, {"act", act}}; }
+  int64_t hidden = 0, intermediate = 0;
+  std::string n_up, n_down, n_act;
+  Tensor w_up, w_down, act;
+};
+
+// The mLSTM cell.  With q = W_q h / sqrt(dk), k = W_k h (heads x dk), v = W_v h (heads x dv) and per head a log
+// input gate i = cap tanh((W_i h + b_i) / cap) and a log forget gate f = logsigmoid(cap tanh((W_f h + b_f) / cap)):
+//   m_t = max(f + m_(t-1), i);  S_t = exp(f + m_(t-1) - m_t) S_(t-1) + exp(i - m_t) k v^T;  n_t likewise with k;
+//   o = S_t^T q / (max(|n_t . q|, exp(-m_t)) + 1e-6),
+// S, n and m starting at zero.  Each head's o is divided by its root mean square, the heads are multiplied by the
+// vector `norm` and by sigmoid(W_g h), and W_o maps them back.  q, k, v, the output gate and the two gates'
+// pre-activations come from one product with the stacked weight [q; k; v; g; i; f].  The memory (S, n, m per head)
+// is per-request state in 32-bit: a request's slot, zeroed when it is admitted; each run of the layer has its own.
+// Tensor names: prefix + ".q", ".k", ".v", ".g", ".o", ".norm", ".i", ".i.b", ".f", ".f.b".
+class MLSTM final : public MixerPart {
+ public:
+  MLSTM(const std::string& prefix, const Json& p) : MixerPart(prefix) {
+    hidden = param_int(p, "hidden");
+    heads = (int)param_int(p, "heads");
+    dk = (int)param_int(p, "head_dim");
+    dv = p.has("v_head_dim") ? (int)param_int(p, "v_head_dim") : dk;
+    cap = (float)param_float(p, "gate_cap");
+    eps = (float)param_float(p, "eps");
+    if (heads <= 0 || dk <= 0 || dv <= 0 || hidden <= 0) throw ConfigError("mlstm: sizes must be positive");
+    if (dk > 256) throw ConfigError("mlstm: a key size of " + std::to_string(dk) + " is not served (up to 256)");
+    const int padded = dk <= 32 ? 32 : dk <= 64 ? 64 : dk <= 128 ? 128 : 256;      // the rows the scan kernel holds
+    if (2 * padded + dv > 1020)
+      throw ConfigError("mlstm: a value size of " + std::to_string(dv) + " beside a key size of " + std::to_string(dk) +
+                        " is not served (the scan stages sixteen tokens' q, k and v in 64 KB)");
+    if (!(cap > 0.f)) throw ConfigError("mlstm: gate_cap must be positive");
+    nq = (int64_t)heads * dk;
+    nv = (int64_t)heads * dv;
+    width = 2 * nq + 2 * nv + 2 * heads;
+  }
+  const char* kind_name() const override { return "mlstm"; }
+  bool reads_through_ops() const override { return true; }
+  bool can_store() const override { return true; }
+  std::string name(const char* t) const { return join(prefix, t); }
+  std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
+    TensorNeed qk, v, o, gate, bias, nw;
+    qk.shape = {nq, hidden};
+    v.shape = {nv, hidden};
+    o.shape = {hidden, nv};
+    gate.shape = {heads, hidden};
+    bias.shape = {heads};
+    bias.role = TensorNeed::Vector;
+    bias.b = 1.0;
+    nw.shape = {nv};
+    nw.role = TensorNeed::Vector;
+    nw.a = 1.0;
+    nw.b = 0.1;
+    return {{name("q"), qk}, {name("k"), qk}, {name("v"), v}, {name("g"), v}, {name("o"), o}, {name("norm"), nw},
+            {name("i"), gate}, {name("i.b"), bias}, {name("f"), gate}, {name("f.b"), bias}};
+  }
+  void load(WeightSource& src) override {
+    w_in = src.alloc(src.matrix_dtype, {width, hidden});
+    src.fill(name("q"), w_in.rows(0, nq));
+    src.fill(name("k"), w_in.rows(nq, nq));
+    src.fill(name("v"), w_in.rows(2 * nq, nv));
+    src.fill(name("g"), w_in.rows(2 * nq + nv, nv));
+    src.fill(name("i"), w_in.rows(2 * nq + 2 * nv, heads));
+    src.fill(name("f"), w_in.rows(2 * nq + 2 * nv + heads, heads));
+    TensorNeed o, bias, nw;
+    o.shape = {hidden, nv};
+    bias.shape = {heads};
+    bias.role = TensorNeed::Vector;
+    nw.shape = {nv};
+    nw.role = TensorNeed::Vector;
+    w_o = src.fetch(name("o"), o);
+    norm_w = src.fetch(name("norm"), nw);
+    b_i = src.fetch(name("i.b"), bias);
+    b_f = src.fetch(name("f.b"), bias);
+  }
+  bool has_cache() const override { return true; }
+  CacheNeed cache_need() const override {
+    CacheNeed n;
+    n.kind = CacheNeed::State;
+    n.state_shape = {heads, (int64_t)dk * dv + dk + 1};
+    return n;
+  }
+  void run(StepContext& ctx, const Rows& h, const Tensor& out, Ops::Epilogue epi) {
+    const int64_t M = h.t.shape[0];
+    Tensor proj = ctx.buf("mlstm.proj", DType::F32, {M, width});
+    ctx.ops.linear(h, w_in, proj, Ops::Store);
+    const auto bound = ctx.binding(this);
+    const Tensor state = ctx.state(bound.first, bound.second);
+    Tensor o = ctx.buf("mlstm.o", DType::F32, {M, nv});
+    Ops::MlstmColumns cols;
+    cols.q = 0;
+    cols.k = (int)nq;
+    cols.v = (int)(2 * nq);
+    cols.i = (int)(2 * nq + 2 * nv);
+    cols.f = cols.i + heads;
+    ctx.ops.mlstm_scan(proj, cols, b_i, b_f, state, ctx.entry_meta, (int)ctx.entries.size(), o, heads, dk, dv, cap,
+                       (float)(1.0 / std::sqrt((double)dk)));
+    Tensor a = ctx.buf("mlstm.gated", ctx.act_dtype, {M, nv});
+    ctx.ops.gated_head_norm(o, proj, (int)(2 * nq + nv), norm_w, eps, a, heads, dv);
+    ctx.ops.linear(a, w_o, out, epi, epi == Ops::Add);
+  }
+  void forward(StepContext& ctx, const Rows& h, const Tensor& x) override { run(ctx, h, x, Ops::Add); }
+  void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override { run(ctx, h, y, Ops::Store); }
+  std::vector<std::pair<std::string, Tensor>> held() const override {
+    return {{"w_in", w_in}, {"w_o", w_o}, {"norm_w", norm_w}, {"b_i", b_i}, {"b_f", b_f}};
+  }
+  int64_t hidden = 0, nq = 0, nv = 0, width = 0;
+  int heads = 0, dk = 0, dv = 0;
+  float cap = 1.f, eps = 1e-6f;
+  Tensor w_in, w_o, norm_w, b_i, b_f;
+};
+
+// A parallel layer: h = norm1(x); x += s1 * mixer(h) + s2 * ffn(h).  One norm feeds both branches; each branch's
+// output is scaled per channel by a learned vector (`scale1`, `scale2`: the tensors' names after the prefix, absent:
+// no scaling) before the two are added to the residual together, in 32-bit.  Without a feed-forward the mixer alone
+// is added.  Branches that can write their output apart from the residual do so; others add into a zeroed buffer.
+class ParallelBlock final : public BlockPart {
+ public:
+  ParallelBlock(const std::string& prefix, const Json& p, const PartChildren& c) : BlockPart(prefix) {
+    for (const auto& kv : c) {
+      if (kv.first == "norm1") norm1 = std::dynamic_pointer_cast<NormPart>(kv.second);
+      if (kv.first == "mixer") mixer = std::dynamic_pointer_cast<MixerPart>(kv.second);
+      if (kv.first == "ffn") ffn = std::dynamic_pointer_cast<FeedForwardPart>(kv.second);
+    }
+    if (!norm1 || !mixer) throw ConfigError("block 'parallel' needs norm1 and mixer parts (ffn is optional)");
+    dim = param_int(p, "dim");
+    if (p.has("scale1")) scale1 = join(prefix, p.at("scale1").as_string());
+    if (p.has("scale2")) scale2 = join(prefix, p.at("scale2").as_string());
+  }
+  const char* kind_name() const override { return "parallel"; }
+  bool reads_through_ops() const override { return true; }
+  std::vector<std::shared_ptr<Part>> children() const override {
+    std::vector<std::shared_ptr<Part>> v = {norm1, mixer};
+    if (ffn) v.push_back(ffn);
+    return v;
+  }
+  std::vector<std::string> child_slots() const override {
+    std::vector<std::string> v = {"norm1", "mixer"};
+    if (ffn) v.push_back("ffn");
+    return v;
+  }
+  std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
+    std::vector<std::pair<std::string, TensorNeed>> t;
+    TensorNeed n;
+    n.shape = {dim};
+    n.role = TensorNeed::Vector;
+    n.a = 1.0;
+    n.b = 0.3;
+    if (!scale1.empty()) t.emplace_back(scale1, n);
+    if (!scale2.empty()) {
+      n.optional = !ffn;     // a layer without a feed-forward has nothing for it to scale
+      t.emplace_back(scale2, n);
+    }
+    return t;
+  }
+  void load(WeightSource& src) override {
+    TensorNeed n;
+    n.shape = {dim};
+    n.role = TensorNeed::Vector;
+    if (!scale1.empty()) s1 = src.fetch(scale1, n);
+    if (!scale2.empty() && ffn) s2 = src.fetch(scale2, n);
+  }
+  void forward(StepContext& ctx, const Tensor& x) override {
+    if (!norm1->reads_through_ops()) ctx.ops.flush();
+    const Rows h = norm1->forward(ctx, x, nullptr, 0, false);
+    const int64_t M = x.shape[0];
+    Tensor y1 = ctx.buf("parallel.y1", DType::F32, {M, dim});
+    if (!mixer->reads_through_ops()) ctx.ops.flush();
+    if (mixer->can_store()) {
+      mixer->forward_store(ctx, h, y1);
+    } else {
+      ctx.ops.fill_zero(y1.data, y1.bytes());
+      mixer->forward(ctx, h, y1);
+    }
+    Tensor y2;
+    if (ffn) {
+      y2 = ctx.buf("parallel.y2", DType::F32, {M, dim});
+      if (!ffn->reads_through_ops()) ctx.ops.flush();
+      if (ffn->can_store()) {
+        ffn->forward_store(ctx, h, y2);
+      } else {
+        ctx.ops.fill_zero(y2.data, y2.bytes());
+        ffn->forward(ctx, h, y2);
+      }
+    }
+    ctx.ops.scaled_add(x, y1, s1, y2, s2);
+  }
+  std::vector<std::pair<std::string, Tensor>> held() const override { return {{"s1", s1}, {"s2", s2}}; }
+  std::shared_ptr<NormPart> norm1;
+  std::shared_ptr<MixerPart> mixer;
+  std::shared_ptr<FeedForwardPart> ffn;
+  int64_t dim = 0;
+  std::string scale1, scale2;
+  Tensor s1, s2;
+};
+
+// x += table[row]: a learned vector onto every token of the step (what a looped run of layers adds before each
+// of its passes: the pass number is the row).  `tensor`: the table's name, [rows, dim]; several such blocks share it.
+class AddVectorBlock final : public BlockPart {
+ public:
+  AddVectorBlock(const std::string& prefix, const Json& p) : BlockPart(prefix) {
+    dim = param_int(p, "dim");
+    rows = param_int(p, "rows");
+    row = param_int(p, "row");
+    name = tensor_name(p, "tensor", prefix, "weight");
+    if (row < 0 || row >= rows) throw ConfigError("block 'add_vector': row " + std::to_string(row) + " is outside its " + std::to_string(rows) + " rows");
+  }
+  const char* kind_name() const override { return "add_vector"; }
+  bool reads_through_ops() const override { return true; }
+  std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
+    TensorNeed n;
+    n.shape = {rows, dim};
+    n.role = TensorNeed::Vector;
+    n.b = 0.5;
+    return {{name, n}};
+  }
+  void load(WeightSource& src) override { table = src.fetch(name, tensors()[0].second); }
+  void forward(StepContext& ctx, const Tensor& x) override { ctx.ops.add_row(x, table.rows(row, 1)); }
+  std::vector<std::pair<std::string, Tensor>> held() const override { return {{"table", table}}; }
+  int64_t dim = 0, rows = 0, row = 0;
+  std::string name;
+  Tensor table;
+};
+
 void register_builtin_parts() {
-  register_part("embedding", "table", [](const std::string& prefix, const Json& p, const PartChildren&) {
-    return std::make_shared<Embedding>(prefix, param_int(p, "vocab"), param_int(p, "dim"));
+  register_part("embedding", "table", [](const std::string& prefix, const Json& p, const PartChildren& c) {
+    return std::make_shared<Embedding>(prefix, p, c);
   });
   register_part("head", "linear", [](const std::string& prefix, const Json& p, const PartChildren&) {
     const Json* t = p.find("tied");
     const int tied = (!t || t->is_null()) ? -1 : (t->as_bool() ? 1 : 0);
-    return std::make_shared<LMHead>(prefix, param_int(p, "vocab"), param_int(p, "dim"), tied, p.at("tied_to").as_string());
+    return std::make_shared<LMHead>(prefix, param_int(p, "vocab"), param_int(p, "dim"), tied,
+                                    p.has("tied_to") ? p.at("tied_to").as_string() : std::string(),
+                                    tensor_name(p, "tensor", prefix, "weight"));
   });
   register_part("norm", "rmsnorm", [](const std::string& prefix, const Json& p, const PartChildren&) {
-    return std::make_shared<RMSNorm>(prefix, param_int(p, "dim"), param_float(p, "eps"));
+    return std::make_shared<RMSNorm>(prefix, param_int(p, "dim"), param_float(p, "eps"), p.has("scalar") && p.at("scalar").as_bool(),
+                                     p.has("tensor") ? p.at("tensor").as_string() : std::string());
   });
   register_part("pos", "rope_neox", [](const std::string& prefix, const Json& p, const PartChildren&) {
     return std::make_shared<RotaryNeox>(prefix, param_int(p, "head_dim"), param_float(p, "theta"));
   });
+  register_part("pos", "sinusoidal", [](const std::string& prefix, const Json& p, const PartChildren&) {
+    return std::make_shared<Sinusoidal>(prefix, param_int(p, "dim"), p.has("base") ? param_float(p, "base") : 10000.0);
+  });
+  register_part("ffn", "dense", [](const std::string& prefix, const Json& p, const PartChildren&) {
+    return std::make_shared<DenseFFN>(prefix, p);
+  });
+  register_part("mixer", "mlstm", [](const std::string& prefix, const Json& p, const PartChildren&) {
+    return std::make_shared<MLSTM>(prefix, p);
+  });
+  register_part("block", "parallel",
+                [](const std::string& prefix, const Json& p, const PartChildren& c) { return std::make_shared<ParallelBlock>(prefix, p, c); },
+                {{"norm1", "norm"}, {"mixer", "mixer"}, {"ffn", "ffn?"}});
+  register_part("block", "add_vector",
+                [](const std::string& prefix, const Json& p, const PartChildren&) { return std::make_shared<AddVectorBlock>(prefix, p); });
   register_part("ffn", "swiglu", [](const std::string& prefix, const Json& p, const PartChildren&) {
     return std::make_shared<SwiGLU>(prefix, param_int(p, "hidden"), param_int(p, "intermediate"));
   });
@@ -821,6 +1253,23 @@ namespace tinyinfer {
 namespace {
 void RotaryNeox::upload(void* dst, const void* src, size_t bytes) {
   if (hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice) != hipSuccess) throw KernelError("rotary: copying the inverse frequencies failed");
+}
+void Sinusoidal::upload(void* dst, const void* src, size_t bytes) {
+  if (hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice) != hipSuccess) throw KernelError("sinusoidal positions: copying the frequencies failed");
+}
+void RMSNorm::spread(const Tensor& one, const Tensor& all, bool on_host) {
+  float g = 0.f;
+  if (on_host) {
+    g = *one.ptr<float>();
+    for (int64_t i = 0; i < all.numel(); ++i) all.ptr<float>()[i] = g;
+    return;
+  }
+  // the number may still be on its way from the file: wait for every stream before reading it back
+  if (hipDeviceSynchronize() != hipSuccess || hipMemcpy(&g, one.data, 4, hipMemcpyDeviceToHost) != hipSuccess)
+    throw KernelError("rmsnorm: reading the scalar gain back failed");
+  std::vector<float> host((size_t)all.numel(), g);
+  if (hipMemcpy(all.data, host.data(), host.size() * 4, hipMemcpyHostToDevice) != hipSuccess)
+    throw KernelError("rmsnorm: spreading the scalar gain failed");
 }
 }  // namespace
 }  // namespace tinyinfer

@@ -39,9 +39,10 @@ def _candidates(config_dict: Mapping[str, Any]):
     archs = config_dict.get("architectures")
     if isinstance(archs, (list, tuple)):
         out.extend(a for a in archs if isinstance(a, str))
-    mt = config_dict.get("model_type")
-    if isinstance(mt, str):
-        out.append(mt)
+    for key in ("model_type", "architecture"):
+        name = config_dict.get(key)
+        if isinstance(name, str):
+            out.append(name)
     return out
 
 

@@ -121,9 +121,13 @@ class PagedKVNeed:
     kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_dim: Optional[int] = None      # the size of a value where it differs from head_dim
 
     def to_dict(self) -> dict:
-        return {"kind": "paged_kv", "kv_heads": self.kv_heads, "head_dim": self.head_dim, "window": self.window}
+        d = {"kind": "paged_kv", "kv_heads": self.kv_heads, "head_dim": self.head_dim, "window": self.window}
+        if self.v_dim:
+            d["v_dim"] = self.v_dim
+        return d
 
 
 @dataclass(frozen=True)
@@ -155,4 +159,4 @@ def cache_need_from_dict(d):
         return StateNeed(tuple(d["shape"]))
     if d["kind"] == "paged_rows":
         return PagedRowsNeed(tuple(d["row_shape"]), bool(d.get("float32")), d.get("window"))
-    return PagedKVNeed(d["kv_heads"], d["head_dim"], d.get("window"))
+    return PagedKVNeed(d["kv_heads"], d["head_dim"], d.get("window"), d.get("v_dim"))
