@@ -1,0 +1,422 @@
+"""Miterax on the GPU against the plain implementation: every mechanism alone through the kernels' own object, and the
+engine under every way of cutting the work (each request whole; most of it in one step and its last tokens one by
+one; portions of changing size down to two tokens; up to four live requests mixed, with so few pages and state
+slots that both are used again), in 32-bit and in bfloat16, and greedy generation through the entry point and the
+scheduler."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import miterax_models as mm
+import traces
+from helpers import random_tokens
+from plain import miterax_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+# rms of (engine - plain) over rms of the plain logits, per position.  float32: rounding of 32-bit sums against float64.
+# bfloat16: operands of every product, cached keys and values and the query are rounded to 8 bits; the looped and
+# gated models amplify that to a few per cent (measured: up to 2 %), while a lost key, gate or state changes tens of per cent.
+# In bfloat16 a few positions are ill-conditioned by the design itself (an mLSTM's first token is v times the sign of k . q
+# after its norm), so there the bound holds for all but 2 % of the positions; 32-bit holds everywhere.
+TOL = {"float32": 1e-4, "bfloat16": 6e-2}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import tinyinfer_amd  # noqa: F401
+    from tinyinfer_amd.ops.kernels import get_ops
+    return get_ops()
+
+
+def dev(a, dtype=torch.float32):
+    return torch.as_tensor(np.asarray(a)).to(dtype).to("cuda")
+
+
+def f64(t):
+    return t.detach().to("cpu", torch.float64).numpy()
+
+
+def bf16_round(a):
+    return torch.as_tensor(np.asarray(a, dtype=np.float32)).to(torch.bfloat16).to(torch.float64).numpy()
+
+
+# ---------------------------------------------------------------------------------- each mechanism alone
+def test_add_sinusoid_and_add_row(ops):
+    H, pos = 37, [0, 1, 63, 64, 1000, 4095]
+    inv = np.array([10000.0 ** (-2.0 * i / H) for i in range((H + 1) // 2)], dtype=np.float32)
+    x0 = np.random.default_rng(1).normal(size=(len(pos), H))
+    x = dev(x0)
+    ops.add_sinusoid(x, dev(pos, torch.int32), dev(inv))
+    # the angle is a 32-bit product: compare with the same angle, its sine and cosine exact
+    want = x0.copy()
+    for m, p in enumerate(pos):
+        for c in range(H):
+            a = float(np.float32(p) * inv[c // 2])
+            want[m, c] += math.sin(a) if c % 2 == 0 else math.cos(a)
+    assert np.abs(f64(x) - want).max() < 2e-6
+    assert np.abs(f64(x) - (x0 + plain.sinusoid(pos, H))).max() < 5e-4      # and near the exact angle
+    v = np.random.default_rng(2).normal(size=(3, H))
+    ops.add_row(x, dev(v)[1])
+    assert np.abs(f64(x) - (want + v[1])).max() < 3e-6
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_xielu(ops, dtype):
+    rng = np.random.default_rng(3)
+    z = np.concatenate([rng.normal(size=500) * 3, [0.0, -1e-4, 1e-4, -20.0, 15.0]]).astype(np.float32)
+    for p, q in [(0.3, -0.7), (-2.0, 1.5), (0.0, 0.0)]:
+        out = torch.empty(len(z), device="cuda", dtype=DT[dtype])
+        ops.xielu(dev(z), dev([p, q]), out)
+        want = plain.xielu(z.astype(np.float64), p, q)
+        tol = 2e-6 * (1 + np.abs(want)) if dtype == "float32" else 2.0 ** -8 * np.abs(want) + 1e-6
+        assert (np.abs(f64(out) - want) <= tol).all()
+
+
+def test_scaled_add(ops):
+    rng = np.random.default_rng(4)
+    x0, a, b = rng.normal(size=(5, 19)), rng.normal(size=(5, 19)), rng.normal(size=(5, 19))
+    sa, sb = rng.normal(size=19), rng.normal(size=19)
+    x = dev(x0)
+    ops.scaled_add(x, dev(a), dev(sa), dev(b), dev(sb))
+    assert np.abs(f64(x) - (x0 + a * sa + b * sb)).max() < 2e-6
+    x = dev(x0)
+    ops.scaled_add(x, dev(a), dev(sa))
+    assert np.abs(f64(x) - (x0 + a * sa)).max() < 2e-6
+
+
+def paged(rng, n_tokens, P, extra_pages=3):
+    """A block table for one request of n_tokens over shuffled pages: (table [1, width], number of pages)."""
+    n_pages = -(-n_tokens // P)
+    ids = rng.permutation(n_pages + extra_pages)[:n_pages]
+    return np.asarray(ids, dtype=np.int32)[None, :], n_pages + extra_pages
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("heads,kv,dk,dv,P", [(4, 2, 16, 24, 16), (3, 3, 7, 9, 4), (6, 1, 40, 33, 64), (2, 2, 256, 130, 16), (2, 1, 64, 64, 16)])
+def test_split_write_and_capped_attention(ops, dtype, heads, kv, dk, dv, P):
+    """q/k/v of a whole request written in two portions, then attention of chosen rows: the first tokens, both sides
+    of every page border, a far row.  One key far back gets a score that stands out, so losing it shows."""
+    rng = np.random.default_rng(dk * 1000 + dv)
+    T, coef, every, scale, cap = 150, 0.4, 5, 1.0 / math.sqrt(dk), 12.0
+    q = rng.normal(size=(T, heads, dk))
+    k = rng.normal(size=(T, kv, dk))
+    v = rng.normal(size=(T, kv, dv))
+    far = 2
+    k[far] *= 3.0                                    # ... and the last query points at it
+    q[T - 1] = k[far][np.arange(heads) // (heads // kv)] / 3.0
+    qkv = np.concatenate([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], axis=1)
+    table, n_pages = paged(rng, T, P)
+    pool = torch.zeros(n_pages, kv, P, dk + dv, device="cuda", dtype=DT[dtype])
+    q_out = torch.empty(T, heads * dk, device="cuda", dtype=DT[dtype])
+    pos = np.arange(T, dtype=np.int32)
+    slots = np.zeros(T, dtype=np.int32)
+    cut = 37
+    for lo, hi in ((0, cut), (cut, T)):
+        ops.qkv_split_write(dev(qkv[lo:hi]), dev(pos[lo:hi], torch.int32), dev(slots[lo:hi], torch.int32), dev(table, torch.int32),
+                            pool, q_out[lo:hi], heads, kv, dk, dv, coef, every)
+    temp = np.array([plain.query_temperature(p, coef, every) for p in range(T)])
+    rnd = (lambda a: a) if dtype == "float32" else bf16_round
+    qt = rnd((q * temp[:, None, None]).astype(np.float32))
+    # bfloat16: the temperature's 32-bit logarithm may round a product the other way: one step of the last place
+    got_q = f64(q_out).reshape(T, heads, dk)
+    assert (np.abs(got_q - qt) <= (1e-6 if dtype == "float32" else 2.0 ** -7) * np.abs(qt) + 1e-30).all()
+    qt = got_q
+    kr, vr = rnd(k), rnd(v)
+    rows = sorted({0, 1, 2, P - 1, P, P + 1, 2 * P - 1, 2 * P, cut - 1, cut, T - 2, T - 1} & set(range(T)))
+    out = torch.empty(len(rows), heads * dv, device="cuda", dtype=DT[dtype])
+    ops.attention_capped(q_out[rows].contiguous(), pool, dev(table, torch.int32), dev(pos[rows], torch.int32),
+                         dev(slots[rows], torch.int32), out, heads, kv, dk, dv, scale, cap)
+    want = np.zeros((len(rows), heads, dv))
+    weight_of_far = 0.0
+    for r, i in enumerate(rows):
+        for h in range(heads):
+            g = h // (heads // kv)
+            s = cap * np.tanh((kr[: i + 1, g] @ qt[i, h]) * scale / cap)
+            p = np.exp(s - s.max())
+            p /= p.sum()
+            want[r, h] = p @ vr[: i + 1, g]
+            if i == T - 1:
+                weight_of_far = max(weight_of_far, p[far])
+    assert weight_of_far > 0.3                       # the far key matters
+    tol = 3e-6 if dtype == "float32" else 1e-2
+    assert np.abs(f64(out).reshape(len(rows), heads, dv) - want).max() < tol * max(1.0, np.abs(want).max())
+
+
+def plain_cell(q, k, v, ig, fg, S, n, m):
+    """One request's tokens through the mLSTM recurrence from (S, n, m); returns o and the new state."""
+    o = np.zeros((q.shape[0], v.shape[1]))
+    for t in range(q.shape[0]):
+        m_new = max(fg[t] + m, ig[t])
+        decay, take = math.exp(fg[t] + m - m_new), math.exp(ig[t] - m_new)
+        S = decay * S + take * np.outer(k[t], v[t])
+        n = decay * n + take * k[t]
+        m = m_new
+        o[t] = (S.T @ q[t]) / (max(abs(float(n @ q[t])), math.exp(-m)) + 1e-6)
+    return o, S, n, m
+
+
+@pytest.mark.parametrize("heads,dk,dv", [(2, 16, 24), (1, 33, 17), (3, 64, 64), (1, 130, 70), (2, 8, 300), (1, 256, 128)])
+def test_mlstm_scan_carries_its_state(ops, heads, dk, dv):
+    """Three requests of unequal length in one step into slots 2, 0 and 3, then each goes on with more tokens (one of
+    them with a single one), then slot 0 is zeroed and used by a new request: every output and the final states against
+    the recurrence from the formulas."""
+    rng = np.random.default_rng(dk + dv)
+    cap = 5.0
+    N = heads * (2 * dk + 2 * dv + 2) + 3                      # some columns the scan does not read
+    cols = dict(q=0, k=heads * dk + 1, v=2 * heads * dk + 1, i=2 * heads * dk + heads * dv + 2, f=2 * heads * dk + heads * dv + 2 + heads)
+    per_head = dk * dv + dk + 1
+    state = torch.zeros(4, heads, per_head, device="cuda")
+    bi, bf = rng.normal(size=heads), rng.normal(size=heads) + 1.5
+    ref = {}                                                   # slot -> per head (S, n, m)
+
+    def step(lengths, slots):
+        M = sum(lengths)
+        proj = rng.normal(size=(M, N)).astype(np.float32)
+        proj[:, cols["i"]:cols["i"] + heads] *= 4.0            # gates that reach their cap
+        entries, row = [], 0
+        for n_tok, s in zip(lengths, slots):
+            entries.append([row, n_tok, 0, s])
+            row += n_tok
+        o = torch.full((M, heads * dv), 7.0, device="cuda")
+        ops.mlstm_scan(dev(proj), dev(bi), dev(bf), state, dev(entries, torch.int32), o, heads, dk, dv, cap, dk ** -0.5,
+                       (cols["q"], cols["k"], cols["v"], cols["i"], cols["f"]))
+        p = proj.astype(np.float64)
+        want = np.zeros((M, heads, dv))
+        for (row0, n_tok, _, s) in entries:
+            for h in range(heads):
+                S, n, m = ref.get((s, h), (np.zeros((dk, dv)), np.zeros(dk), 0.0))
+                rows = slice(row0, row0 + n_tok)
+                q = p[rows, cols["q"] + h * dk: cols["q"] + (h + 1) * dk] * np.float64(np.float32(dk ** -0.5))
+                k = p[rows, cols["k"] + h * dk: cols["k"] + (h + 1) * dk]
+                v = p[rows, cols["v"] + h * dv: cols["v"] + (h + 1) * dv]
+                ig = cap * np.tanh((p[rows, cols["i"] + h] + bi[h]) / cap)
+                fg = plain.logsigmoid(cap * np.tanh((p[rows, cols["f"] + h] + bf[h]) / cap))
+                want[rows, h], S, n, m = plain_cell(q, k, v, ig, fg, S, n, m)
+                ref[(s, h)] = (S, n, m)
+        got = f64(o).reshape(M, heads, dv)
+        assert np.abs(got - want).max() < 2e-4 * max(1.0, np.abs(want).max())
+
+    step([19, 2, 40], [2, 0, 3])
+    step([1, 33, 5], [3, 2, 0])
+    state[0].zero_()
+    for h in range(heads):
+        ref.pop((0, h), None)
+    step([7, 1], [0, 2])
+    st = f64(state)
+    for (s, h), (S, n, m) in ref.items():
+        assert np.abs(st[s, h, : dk * dv].reshape(dk, dv) - S).max() < 2e-4 * max(1.0, np.abs(S).max())
+        assert np.abs(st[s, h, dk * dv: dk * dv + dk] - n).max() < 2e-4 * max(1.0, np.abs(n).max())
+        assert abs(st[s, h, -1] - m) < 1e-5
+    assert float(state[1].abs().max()) == 0.0                  # a slot nobody used stays untouched
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gated_head_norm(ops, dtype):
+    rng = np.random.default_rng(8)
+    M, heads, dv, eps, col = 6, 3, 21, 1e-5, 4
+    o = rng.normal(size=(M, heads * dv)) * 5
+    proj = rng.normal(size=(M, col + heads * dv + 2)) * 2
+    w = rng.normal(size=heads * dv)
+    out = torch.empty(M, heads * dv, device="cuda", dtype=DT[dtype])
+    ops.gated_head_norm(dev(o), dev(proj), col, dev(w), eps, out, heads, dv)
+    want = plain.rms_unit(o.reshape(M, heads, dv), eps).reshape(M, -1) * w * plain.sigmoid(proj[:, col: col + heads * dv])
+    tol = 3e-6 if dtype == "float32" else 2.0 ** -8
+    assert np.abs(f64(out) - want).max() < tol * max(1.0, np.abs(want).max())
+
+
+# --------------------------------------------------------------------------------------- the engine
+REQUEST_LENGTHS = {"a": 97, "b": 45, "c": 130, "d": 33, "e": 71, "f": 58}
+PROMPT_LENGTHS = {"a": 60, "b": 12, "c": 101, "d": 30, "e": 2, "f": 41}
+_made = {}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    def get(name):
+        if name not in _made:
+            config = mm.CONFIGS[name]
+            weights = mm.draw_weights(config, seed=len(name) * 17 + 1)
+            path = mm.write_folder(str(tmp_path_factory.mktemp("miterax_" + name)), config, 0, weights)
+            requests = {r: random_tokens(n, config["vocab"], 7 + i) for i, (r, n) in enumerate(REQUEST_LENGTHS.items())}
+            w = mm.as_float64(weights)
+            want = {r: plain.forward(config, w, t) for r, t in requests.items()}
+            _made[name] = (path, requests, want, w)
+        return _made[name]
+    return get
+
+
+def build_engine(folder, dtype, max_tokens, page_size=16, max_requests=4):
+    import tinyinfer_amd  # noqa: F401
+    from tinyinfer_amd.engine import Engine
+    return Engine.from_folder(folder, dtype, page_size=page_size, max_tokens=max_tokens, max_requests=max_requests, max_seq=max_tokens)
+
+
+def replay(engine, trace):
+    from tinyinfer_amd.engine import StepEntry
+    got = {}
+    for step in trace:
+        logits = engine.step([StepEntry(r, t, w) for r, t, w in step["entries"]])
+        rows = None if logits is None else logits.cpu().numpy().astype(np.float64)
+        i = 0
+        for r, _, w in step["entries"]:
+            for _ in w:
+                got.setdefault(r, []).append(rows[i])
+                i += 1
+        for r in step["end"]:
+            engine.release(r)
+        engine.cache.check()
+    return {r: np.stack(v) for r, v in got.items()}
+
+
+def worst(got, want):
+    """The largest rms(engine - plain) / rms(plain) over all positions, the mean over the vocabulary taken off both."""
+    w, where = 0.0, None
+    for r in want:
+        e = errors(got[r], want[r])
+        if e.max() > w:
+            w, where = float(e.max()), (r, int(e.argmax()))
+    return w, where
+
+
+def errors(got, want):
+    assert got.shape == want.shape, (got.shape, want.shape)
+    d = got - want
+    d = d - d.mean(axis=1, keepdims=True)
+    ref = want - want.mean(axis=1, keepdims=True)
+    return np.sqrt((d ** 2).mean(axis=1)) / np.sqrt((ref ** 2).mean(axis=1))
+
+
+def within(got, want, dtype):
+    """32-bit: every position within the bound.  bfloat16: all but 2 % of them."""
+    if dtype == "float32":
+        w, where = worst(got, want)
+        return w < TOL[dtype], (w, where)
+    e = np.concatenate([errors(got[r], want[r]) for r in want])
+    over = float((e > TOL[dtype]).mean())
+    return over <= 0.02, (over, float(np.median(e)), float(e.max()))
+
+
+def make_trace(mode, requests):
+    if mode == "whole":
+        return traces.whole(requests)
+    if mode == "tail":
+        return traces.tail_one_by_one(requests, 32)
+    if mode == "portions":
+        return traces.portions(requests)
+    return traces.mixed(requests, PROMPT_LENGTHS, live=4)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,page_size", [("loop3", 16), ("noloop", 4), ("wide", 16), ("odd", 32)])
+@pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
+def test_engine_matches_plain(folders, name, page_size, dtype, mode):
+    folder, requests, want, _ = folders(name)
+    trace = make_trace(mode, requests)
+    n_tok = traces.max_pages(trace, page_size) * page_size      # the tightest pool: pages are handed out again
+    engine = build_engine(folder, dtype, n_tok, page_size)
+    got = replay(engine, trace)
+    assert not engine.cache.live_requests()
+    ok, seen = within(got, want, dtype)
+    assert ok, (name, mode, dtype, seen)
+
+
+@pytest.mark.parametrize("name", ["loop3", "odd"])
+def test_cuts_agree_bit_for_bit_in_float32(folders, name):
+    """Token by token from the first token on, in portions, and whole: in 32-bit every sum is taken in an order that does
+    not depend on the step, so the logits are the same bits."""
+    folder, requests, _, _ = folders(name)
+    some = {r: requests[r][:40] for r in ("b", "d")}
+    results = []
+    for trace in (traces.whole(some), traces.tail_one_by_one(some, 39), traces.portions(some), traces.mixed(some, {"b": 20, "d": 3}, live=2)):
+        engine = build_engine(folder, "float32", 256)
+        results.append(replay(engine, trace))
+    for other in results[1:]:
+        for r in some:
+            assert np.array_equal(results[0][r], other[r]), r
+
+
+def test_a_state_slot_used_again_starts_from_zero(folders):
+    """One slot only: the second request gets the slot (and the pages) the first one gave back."""
+    folder, requests, want, _ = folders("noloop")
+    engine = build_engine(folder, "float32", 192, max_requests=1)
+    for r in ("c", "b", "c"):
+        got = replay(engine, traces.portions({r: requests[r]}))
+        w, where = worst(got, {r: want[r]})
+        assert w < TOL["float32"], (r, w, where)
+
+
+def test_long_context_and_long_decoding(folders):
+    """A prompt of 700 tokens in portions of 256, then 200 tokens one by one (the query temperature passes many steps, the
+    recurrent state is carried through all of them), with pages of 64."""
+    folder, _, _, w = folders("loop3")
+    config = mm.CONFIGS["loop3"]
+    toks = random_tokens(900, config["vocab"], 99)
+    want = plain.forward(config, w, toks)
+    engine = build_engine(folder, "float32", 960, page_size=64)
+    from tinyinfer_amd.engine import StepEntry
+    rows, at = [], 0
+    while at < 700:
+        n = min(256, 700 - at)
+        rows.append(engine.step([StepEntry("x", toks[at:at + n], list(range(n)))]).cpu().numpy())
+        at += n
+    for t in toks[700:]:
+        rows.append(engine.step([StepEntry("x", [t], [0])]).cpu().numpy())
+    got = np.concatenate(rows).astype(np.float64)
+    worst_err, where = worst({"x": got}, {"x": want})
+    assert worst_err < 3e-4, (worst_err, where)
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_greedy_generation_through_the_entry_point(folders, use_graph):
+    """Several prompts of unequal length at once through LLM.generate: the scheduler cuts the prompts into portions of 16
+    and batches decoding requests; every generated token is the plain model's argmax."""
+    import tinyinfer_amd as ti
+    folder, requests, _, w = folders("loop3")
+    config = mm.CONFIGS["loop3"]
+    prompts = [requests["b"][:37], requests["d"][:5], requests["e"][:50], requests["f"][:1]]
+    n_new = 12
+    llm = ti.LLM(folder, dtype="float32", max_seq=128, max_requests=3, chunk_size=16, max_batched_tokens=40, use_graph=use_graph)
+    got = llm.generate(prompts, max_new_tokens=n_new, temperature=0.0)
+    for p, g in zip(prompts, got):
+        toks = list(p)
+        for _ in range(n_new):
+            logits = plain.forward(config, w, toks)[-1]
+            best = int(np.argmax(logits))
+            margin = logits[best] - np.partition(logits, -2)[-2]
+            toks.append(best)
+            if margin < 1e-3:          # a tie within rounding: what follows may differ legitimately
+                break
+        n = len(toks) - len(p)
+        assert g[:n] == toks[len(p):], (p[:3], g, toks[len(p):])
+
+
+def test_trace_replay_program(folders, tmp_path):
+    """The replay program on a Miterax folder: it picks the model by config.json and writes the logits the engine gives."""
+    import os
+    import subprocess
+    import sys
+    folder, requests, want, _ = folders("odd")
+    some = {r: requests[r] for r in ("b", "d", "f")}
+    trace = traces.mixed(some, PROMPT_LENGTHS, live=2)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out", str(out),
+                           "--max-tokens", str(traces.max_tokens(trace))], input=traces.to_jsonl(trace), text=True,
+                          capture_output=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    V = mm.CONFIGS["odd"]["vocab"]
+    got = {}
+    for i, step in enumerate(trace):
+        assert f"done {i}" in proc.stdout
+        rows = np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, V).astype(np.float64)
+        k = 0
+        for r, _, wnt in step["entries"]:
+            for _ in wnt:
+                got.setdefault(r, []).append(rows[k])
+                k += 1
+    w, where = worst({r: np.stack(v) for r, v in got.items()}, {r: want[r] for r in some})
+    assert w < TOL["float32"], (w, where)

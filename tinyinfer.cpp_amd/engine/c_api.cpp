@@ -1222,6 +1222,36 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
                                             arg(1), num(14) != 0, arg(3), (int)num(0), (int)num(1), (int)num(2), (float)num(3),
                                             (int)num(4)));
     }
+  } else if (op == "add_sinusoid") {
+    ops.add_sinusoid(arg(0), iptr(1), arg(2));
+  } else if (op == "add_row") {
+    ops.add_row(arg(0), arg(1));
+  } else if (op == "xielu") {
+    ops.xielu(arg(0), arg(1), arg(2));
+  } else if (op == "scaled_add") {
+    // x, a, scale of a, b, scale of b (the last two or the scales may be absent)
+    ops.scaled_add(arg(0), arg(1), n_t > 2 ? arg(2) : Tensor(), n_t > 3 ? arg(3) : Tensor(), n_t > 4 ? arg(4) : Tensor());
+  } else if (op == "qkv_split_write") {
+    // qkv, positions, slots, table, pool [pages, kv_heads, P, dk + dv], q_out; heads, kv_heads, dk, dv, coef, every
+    ops.qkv_split_write(arg(0), iptr(1), iptr(2), view_of(3, arg(4)), arg(4), arg(5), (int)num(0), (int)num(1), (int)num(2),
+                        (int)num(3), (float)num(4), (int)num(5));
+  } else if (op == "attention_capped") {
+    // q, pool, table, positions, slots, out; heads, kv_heads, dk, dv, scale, softcap, window
+    ops.attention_capped(arg(0), arg(1), view_of(2, arg(1)), iptr(3), iptr(4), arg(5), (int)num(0), (int)num(1), (int)num(2),
+                         (int)num(3), (float)num(4), (float)num(5), (int)num(6));
+  } else if (op == "mlstm_scan") {
+    // proj, bias_i, bias_f, state, entries [R, 4], o; heads, dk, dv, cap, q_scale, columns of q, k, v, i, f
+    Ops::MlstmColumns c;
+    c.q = (int)num(5);
+    c.k = (int)num(6);
+    c.v = (int)num(7);
+    c.i = (int)num(8);
+    c.f = (int)num(9);
+    ops.mlstm_scan(arg(0), c, arg(1), arg(2), arg(3), iptr(4), (int)arg(4).shape[0], arg(5), (int)num(0), (int)num(1), (int)num(2),
+                   (float)num(3), (float)num(4));
+  } else if (op == "gated_head_norm") {
+    // o, proj, w, out; gate column, eps, heads, dv
+    ops.gated_head_norm(arg(0), arg(1), (int)num(0), arg(2), (float)num(1), arg(3), (int)num(2), (int)num(3));
   } else if (op == "argmax") {
     ops.argmax(arg(0), arg(1).ptr<int>());
   } else if (op == "sample") {

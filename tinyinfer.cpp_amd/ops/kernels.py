@@ -94,7 +94,9 @@ _SWITCHES = {"use_fast_gemm": "fast_gemm", "use_fast_attention": "fast_attention
              "use_radix_sample": "radix_sample"}
 _LIB_OF = {"embed": "core", "rmsnorm": "core", "rope_neox": "core", "rope_table": "core", "qk_norm_rope_kv_write": "core",
            "qk_norm_inplace": "core", "argmax": "sampling", "sample": "sampling", "attention_rows": "attention_generic",
-           "fill_random": "core", "fill_zero": "core"}
+           "fill_random": "core", "fill_zero": "core", "add_sinusoid": "pointwise", "add_row": "pointwise", "xielu": "pointwise",
+           "scaled_add": "pointwise", "qkv_split_write": "pointwise", "attention_capped": "attention_generic",
+           "mlstm_scan": "recurrent", "gated_head_norm": "recurrent"}
 
 
 class Ops:
@@ -315,6 +317,37 @@ class Ops:
                                fold=(1,), libs=["attention_bf16", "core"]))
 
     # ------------------------------------------------------------------ sampling
+    # ---- layers beyond the pre-norm transformer block
+    def add_sinusoid(self, x, positions, inv_freq):
+        """x f32 [M, H]: x[m, 2i] += sin(pos[m] inv_freq[i]), x[m, 2i + 1] += cos(the same)."""
+        self._call("add_sinusoid", [x, positions, inv_freq])
+
+    def add_row(self, x, v):
+        self._call("add_row", [x, v])
+
+    def xielu(self, z, act, out):
+        """out = xIELU(z) with act = (p, q), z float32."""
+        self._call("xielu", [z, act, out])
+
+    def scaled_add(self, x, a, sa=None, b=None, sb=None):
+        """x += a * sa + b * sb per channel."""
+        self._call("scaled_add", [x, a, sa, b, sb])
+
+    def qkv_split_write(self, qkv, positions, slots, table, pool, q_out, heads, kv_heads, dk, dv, coef=0.0, every=1):
+        """qkv f32 [M, heads dk + kv_heads (dk + dv)]; pool [pages, kv_heads, P, dk + dv] (a page: K [kv][P][dk] | V [kv][dv][P])."""
+        self._call("qkv_split_write", [qkv, positions, slots, table, pool, q_out], [heads, kv_heads, dk, dv, coef, every])
+
+    def attention_capped(self, q, pool, table, positions, slots, out, heads, kv_heads, dk, dv, scale, softcap=0.0, window=0):
+        self._call("attention_capped", [q, pool, table, positions, slots, out],
+                   [heads, kv_heads, dk, dv, scale, softcap, int(window or 0)])
+
+    def mlstm_scan(self, proj, bias_i, bias_f, state, entries, o, heads, dk, dv, cap, q_scale, columns):
+        """entries int32 [R, 4] = (first row, tokens, -, state slot); columns = (q, k, v, i, f) of proj."""
+        self._call("mlstm_scan", [proj, bias_i, bias_f, state, entries, o], [heads, dk, dv, cap, q_scale] + list(columns))
+
+    def gated_head_norm(self, o, proj, gate_col, w, eps, out, heads, dv):
+        self._call("gated_head_norm", [o, proj, w, out], [gate_col, eps, heads, dv])
+
     def argmax(self, logits, out):
         if out.dtype != native.torch().int32 or out.shape[0] < logits.shape[0]:
             raise KernelError("argmax: logits must be contiguous float32 [n, V], out int32 [n]")
