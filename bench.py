@@ -18,6 +18,15 @@ as the reference times its own kernels against the clock
 `--model 8b` and `--model 32b` run the same with the sizes of Qwen3-8B and
 Qwen3-32B.  `--kernel-times` adds a table of the decode step's calls, timed with
 events (a line of its own on stderr).
+
+`--design miterax` runs the same measurements on a Miterax decoder whose layers have
+the widths of `--model` (residual width, heads, kv heads, head size 128 for keys and
+values, feed-forward width, vocabulary, number of layers): parallel layers with a
+dense xIELU feed-forward, and as mixers `--mixers attention` (capped attention in
+every layer), `mlstm` (an mLSTM in every layer, as many heads as the model has kv
+heads) or `alternate` (attention, mLSTM, attention, ...).  Run it beside the default
+design with the same `--model` and `--layers`; the default workload and its line stay
+as they are.
 """
 from __future__ import annotations
 
@@ -45,6 +54,23 @@ MODELS = {
                 intermediate_size=25600, tie_word_embeddings=False),
 }
 NAMES = {"0.6b": "Qwen3-0.6B", "1.7b": "Qwen3-1.7B", "4b": "Qwen3-4B", "8b": "Qwen3-8B", "14b": "Qwen3-14B", "32b": "Qwen3-32B"}
+
+
+def miterax_config(base, mixers):
+    """A Miterax config.json with the layer widths of the Qwen3 configuration `base`."""
+    H, F = base["hidden_size"], base["intermediate_size"]
+    attention = dict(type="attention", mixer=dict(heads=base["num_attention_heads"], kv_heads=base["num_key_value_heads"],
+                                                  dim=base["head_dim"], vdim=base["head_dim"], scale=base["head_dim"] ** -0.5,
+                                                  softcap=30.0, q_temp=dict(coef=0.1, every=256)),
+                     mlp=dict(kind="dense", ff=F))
+    mlstm = dict(type="mlstm", mixer=dict(heads=base["num_key_value_heads"], dim=base["head_dim"], vdim=base["head_dim"], gate_cap=15.0),
+                 mlp=dict(kind="dense", ff=F))
+    kinds = {"attention": [attention], "mlstm": [mlstm], "alternate": [attention, mlstm]}[mixers]
+    L = base["num_hidden_layers"]
+    return dict(architecture="Miterax", width=H, vocab=base["vocab_size"], norm=dict(eps=1e-6),
+                layers=[kinds[i % len(kinds)] for i in range(L)])
+
+
 MAX_SEQ = 4096            # context length a request may reach (more if --context asks for it)
 PAGE = 16
 PEAK_HBM = 8.0e12         # bytes/s, MI355X
@@ -63,6 +89,7 @@ def model_numbers(model):
     seen = set()
     layer_params = head_params = vector_params = embed_row = 0
     attn = []                     # (heads, head_dim, window) of every mixer that attends over cached keys
+    cells = []                    # shape of the per-request state of every recurrent mixer
     for part in model.parts():
         for name, need in part.tensors().items():
             n = 1
@@ -83,17 +110,32 @@ def model_numbers(model):
         need = part.cache_need()
         if need is not None and hasattr(need, "kv_heads") and "heads" in getattr(part, "params", {}):
             attn.append((part.params["heads"], need.head_dim, need.window))
+        if need is not None and hasattr(need, "shape") and not hasattr(need, "kv_heads"):
+            cells.append(tuple(need.shape))
     weight_bytes = (layer_params + head_params) * 2 + vector_params * 4 + embed_row * 2
-    kv_bytes = lambda context: sum(2 * need.kv_heads * need.head_dim * 2 * n * min(context, need.window or context)      # noqa: E731
-                                   for need, n in model.cache_groups if hasattr(need, "kv_heads"))
-    return dict(layer_params=layer_params, head_params=head_params, weight_bytes=weight_bytes, kv_bytes=kv_bytes, attention=attn)
+    # per cached token the keys and values of every cache layer (values of their own size where they have one); per
+    # request the 32-bit state of every recurrent layer, read and written once a step
+    state_bytes = sum(2 * 4 * int(np_prod(need.shape)) * n for need, n in model.cache_groups if not hasattr(need, "kv_heads") and hasattr(need, "shape"))
+    kv_bytes = lambda context: state_bytes + sum(need.kv_heads * (need.head_dim + (getattr(need, "v_dim", None) or need.head_dim)) * 2 * n *      # noqa: E731
+                                                 min(context, need.window or context)
+                                                 for need, n in model.cache_groups if hasattr(need, "kv_heads"))
+    return dict(layer_params=layer_params, head_params=head_params, weight_bytes=weight_bytes, kv_bytes=kv_bytes, attention=attn,
+                cells=cells, state_bytes=state_bytes)
+
+
+def np_prod(shape):
+    n = 1
+    for d in shape:
+        n *= d
+    return n
 
 
 def prefill_flops(model, T):
     n = model_numbers(model)
     gemm = 2.0 * n["layer_params"] * T + 2.0 * n["head_params"]              # the head runs on one row
     attn = sum(2.0 * hd * T * (T + 1) * heads for heads, hd, _ in n["attention"])   # QK^T and PV over the causal half
-    return gemm + attn
+    cells = sum(6.0 * np_prod(shape) * T for shape in n["cells"])                   # decay, outer product and read-out of a memory
+    return gemm + attn + cells
 
 
 def measured_peaks():
@@ -149,6 +191,8 @@ def decode_floor(engine, rids, last, nums, context, batch):
     for c in calls:
         m = re.search(r"\* (\d+)x(\d+)", c["name"])
         per_call = int(m.group(1)) * int(m.group(2)) * 2 if m else kv_layer if c["name"].startswith("attention") else 4096
+        if c["name"].startswith("mlstm_scan") and nums["cells"]:
+            per_call = 2 * 4 * np_prod(nums["cells"][0]) * batch      # the requests' state, read and written
         sizes += [per_call] * c["calls"]
         if c["name"].startswith("attention") and "runs" in c["name"]:
             sizes += [4096] * c["calls"]              # the kernel that merges the runs of a context
@@ -322,6 +366,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--model", choices=sorted(MODELS), default="0.6b", help="whose layer sizes the model has")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
+    ap.add_argument("--design", choices=["qwen3", "miterax"], default="qwen3",
+                    help="miterax: a Miterax decoder with the layer widths of --model instead (see --mixers)")
+    ap.add_argument("--mixers", choices=["attention", "mlstm", "alternate"], default="alternate",
+                    help="--design miterax: the mixer of its layers")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048, help="cached tokens each decoding request holds")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
@@ -351,6 +399,10 @@ def main() -> int:
     layers_full = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
+    sizes, model_name = cfg, f"{NAMES[args.model]} sizes"
+    if args.design == "miterax":
+        cfg = miterax_config(cfg, args.mixers)
+        model_name = f"Miterax ({args.mixers} mixers) at {NAMES[args.model]} sizes"
     rng = np.random.default_rng(0)
     context, prefill_tokens = args.context, args.prefill_tokens
     max_seq = max(MAX_SEQ, context + args.warmup + args.steps + 64, prefill_tokens, args.cached + args.portion)
@@ -360,7 +412,7 @@ def main() -> int:
         say("what the GPU delivers: a kernel that only reads, MFMAs on registers ...")
         peaks = measured_peaks()
         say(f"  read {peaks[0] / 1e9:.0f} GB/s, bf16 MFMA {peaks[1] / 1e12:.0f} TFLOP/s")
-    say(f"building the model ({NAMES[args.model]} sizes, random weights on the device) ...")
+    say(f"building the model ({model_name}, random weights on the device) ...")
     engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", page_size=PAGE,
                                 max_tokens=biggest * (context + 512) + prefill_tokens + args.cached + args.portion,
                                 max_requests=biggest + 1, max_seq=max_seq)
@@ -374,7 +426,7 @@ def main() -> int:
         print(json.dumps({"mixed": {"ms_per_step": round(ms, 3), "host_ms": round(host_ms, 3), "ms_from_graph": round(g_ms, 3),
                                     "host_ms_from_graph": round(g_host, 3), "tokens": args.batch + args.portion,
                                     "decoded": args.batch, "portion": args.portion, "cached": args.cached,
-                                    "decode_context": context, "model": NAMES[args.model]}}), flush=True)
+                                    "decode_context": context, "model": model_name}}), flush=True)
         return 0
     p_s = tps = ms = floor = None
     draw = (args.temperature, args.top_k, args.top_p) if args.temperature > 0 else None
@@ -421,15 +473,15 @@ def main() -> int:
         if peaks:
             prefill.update(measured_mfma_tflops=round(peaks[1] / 1e12, 1), frac_of_measured=round(flops / p_s / peaks[1], 4))
     out = {
-        "metric": f"decode tok/s @ batch {args.batch} ({NAMES[args.model]} sizes, {context:,} cached tokens per request)",
+        "metric": f"decode tok/s @ batch {args.batch} ({model_name}, {context:,} cached tokens per request)",
         "value": None if tps is None else round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": None if ms is None else round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic (uniform random token ids, random weights N(0, 0.02))",
-        "config": {"model": f"{NAMES[args.model]} sizes", "layers": cfg["num_hidden_layers"], "layers_in_config": layers_full,
-                   "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
-                   "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
-                   "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
-                   "tied_head": bool(cfg["tie_word_embeddings"]),
+        "config": {"model": model_name, "layers": sizes["num_hidden_layers"], "layers_in_config": layers_full,
+                   "hidden": sizes["hidden_size"], "heads": sizes["num_attention_heads"],
+                   "kv_heads": sizes["num_key_value_heads"], "head_dim": sizes["head_dim"],
+                   "intermediate": sizes["intermediate_size"], "vocab": sizes["vocab_size"],
+                   "tied_head": bool(sizes["tie_word_embeddings"]) and args.design == "qwen3",
                    "global_batch": args.batch, "cached_tokens": context, "seq_len": max_seq, "page_size": PAGE,
                    "prefill_tokens": prefill_tokens, "parallelism": "single GPU", "decode_graph": True,
                    "sampling": f"temperature {args.temperature} top-k {args.top_k or 512} top-p {args.top_p}" if draw else "greedy"},

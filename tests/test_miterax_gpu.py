@@ -146,6 +146,54 @@ def test_split_write_and_capped_attention(ops, dtype, heads, kv, dk, dv, P):
     assert np.abs(f64(out).reshape(len(rows), heads, dv) - want).max() < tol * max(1.0, np.abs(want).max())
 
 
+@pytest.mark.parametrize("nh,nkv,hd,P", [(4, 2, 64, 16), (8, 2, 128, 16), (6, 3, 32, 16), (3, 1, 128, 32), (2, 2, 48, 16)])
+def test_capped_attention_through_the_step_dispatch(ops, nh, nkv, hd, P):
+    """Keys and values of one size: a step's portions and single tokens go to the matrix-core kernels where they serve the
+    head size (else row by row), with the cap inside.  Scores are large enough for the cap to bend most of them."""
+    from test_kernels_gpu import FakeCtx, View
+    rng = np.random.default_rng(hd + nh)
+    entries = [(200, 0), (1, 300), (70, 130), (1, 15), (33, 1000), (1, 0), (2, 63)]
+    cap, scale = 4.0, 1.0 / math.sqrt(hd)
+    lens = [s + n for n, s in entries]
+    n_pages = [-(-L // P) for L in lens]
+    pages = sum(n_pages) + 5
+    perm = rng.permutation(pages)
+    pool = torch.zeros(pages, 2, nkv, P, hd, dtype=torch.bfloat16)
+    vt = pool[:, 1].reshape(pages, nkv, hd, P)
+    table = np.full((len(entries), max(n_pages) + 1), -1, dtype=np.int32)
+    qs, want, used = [], [], 0
+    for e, ((n, start), L) in enumerate(zip(entries, lens)):
+        q = bf16_round(rng.normal(size=(L, nh, hd)) * 2.0)
+        k = bf16_round(rng.normal(size=(L, nkv, hd)))
+        v = bf16_round(rng.normal(size=(L, nkv, hd)))
+        mine = perm[used:used + n_pages[e]]
+        used += n_pages[e]
+        table[e, :len(mine)] = mine
+        for t in range(L):
+            pool[mine[t // P], 0, :, t % P] = torch.as_tensor(k[t]).to(torch.bfloat16)
+            vt[mine[t // P], :, :, t % P] = torch.as_tensor(v[t]).to(torch.bfloat16)
+        for i in range(start, L):
+            row = []
+            for h in range(nh):
+                g = h // (nh // nkv)
+                s = cap * np.tanh((k[: i + 1, g] @ q[i, h]) * scale / cap)
+                p = np.exp(s - s.max())
+                row.append((p / p.sum()) @ v[: i + 1, g])
+            want.append(np.concatenate(row))
+        qs.append(q[start:])
+    qd = dev(np.concatenate(qs).reshape(-1, nh * hd), torch.bfloat16)
+    out = torch.zeros_like(qd)
+    ctx = FakeCtx(entries)
+    ops.count_calls(True)
+    ops.attention(ctx, View(dev(table, torch.int32)), qd, pool.to("cuda"), out, nh, nkv, hd, scale, None, softcap=cap)
+    names = [r["name"] for r in ops.timing_report()]
+    ops.count_calls(False)
+    assert any(("[mfma]" if hd in (32, 64, 128) else "[generic]") in n for n in names), names
+    want = np.stack(want)
+    assert np.isfinite(f64(out)).all()
+    assert np.abs(f64(out) - want).max() < 2e-2
+
+
 def plain_cell(q, k, v, ig, fg, S, n, m):
     """One request's tokens through the mLSTM recurrence from (S, n, m); returns o and the new state."""
     o = np.zeros((q.shape[0], v.shape[1]))

@@ -107,15 +107,23 @@ struct BlockInfo {
   bool check;   // true: some key of it may be hidden from some column, or not written yet
 };
 
+// tanh from one exponential and one reciprocal: 1 - 2 / (1 + e^(2x)); exact at both ends (e^(2x) = 0 or infinite), within
+// 2e-7 elsewhere, which a soft cap multiplies by the cap: far below a score's own rounding
+__device__ __forceinline__ float tanh_fast(float x) {
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * 2.8853900817779268f));
+}
+
 // One pair of blocks for this wavefront's 16 columns.
 //   qf       Q^T fragments: column lane % 16, dims 32 * step + 8 * (lane / 16) .. + 7
 //   scale    softmax scale times log2(e): scores, maxima and partial maxima are in units of log 2,
 //            so that the weights are bare exp2
 //   lo, hi   the keys this lane's column may see: lo <= key <= hi
 //   kv_last  last position of the request that has been written (rows after it hold rubbish)
+//   cap2     > 0: scores are soft-capped, s <- cap tanh(s / cap), cap2 being the cap in units of log 2 like `scale`
 template <int HD>
 __device__ __forceinline__ void attend_pair(KVPair<HD>& f, const Frag8* qf, BlockInfo A, BlockInfo B, int lo,
-                                            int hi, int kv_last, float scale, float& m, float& l, floatx4* o) {
+                                            int hi, int kv_last, float scale, float& m, float& l, floatx4* o,
+                                            float cap2 = 0.f) {
   const int lane = threadIdx.x & 63;
   const int quad = lane >> 4;
   // S^T = K . Q^T, both blocks
@@ -124,6 +132,14 @@ __device__ __forceinline__ void attend_pair(KVPair<HD>& f, const Frag8* qf, Bloc
   for (int s = 0; s < HD / 32; ++s) {
     sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[0][s].v, qf[s].v, sa, 0, 0, 0);
     sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[1][s].v, qf[s].v, sb, 0, 0, 0);
+  }
+  if (cap2 > 0.f) {      // the same in every lane; before the masks, which put -inf where a key is hidden
+    const float r = scale / cap2, back = cap2 / scale;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      sa[i] = tanh_fast(sa[i] * r) * back;
+      sb[i] = tanh_fast(sb[i] * r) * back;
+    }
   }
   // this lane: keys key0 + 4 quad + i of column lane % 16, in each block
   float sv[8];
@@ -206,7 +222,7 @@ template <int HD, typename Check, typename AfterTable = NoHook, typename BeforeA
 __device__ __forceinline__ void walk_blocks(const PagedKV& kv, const Frag8* qf, int first, int stride, int n,
                                             int lo, int hi, int kv_last, float scale, Check check, float& m,
                                             float& l, floatx4* o, AfterTable after_table = NoHook{},
-                                            BeforeAttend before_attend = NoHook{}) {
+                                            BeforeAttend before_attend = NoHook{}, float cap2 = 0.f) {
   const int lane = threadIdx.x & 63;
   bool hooks_due = true;
   for (int c0 = 0; c0 < n; c0 += 64) {
@@ -241,9 +257,9 @@ __device__ __forceinline__ void walk_blocks(const PagedKV& kv, const Frag8* qf, 
     }
     for (int i = 0; i < nc; i += 4) {
       issue(i + 2, f1, a1, b1);
-      attend_pair<HD>(f0, qf, a0, b0, lo, hi, kv_last, scale, m, l, o);
+      attend_pair<HD>(f0, qf, a0, b0, lo, hi, kv_last, scale, m, l, o, cap2);
       issue(i + 4, f0, a0, b0);
-      if (i + 2 < nc) attend_pair<HD>(f1, qf, a1, b1, lo, hi, kv_last, scale, m, l, o);
+      if (i + 2 < nc) attend_pair<HD>(f1, qf, a1, b1, lo, hi, kv_last, scale, m, l, o, cap2);
     }
   }
   if (hooks_due) {
@@ -378,7 +394,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
                    int table_stride, const int* __restrict__ pos, const int* __restrict__ slot,
                    const int* __restrict__ rows, bf16_t* __restrict__ out, float* __restrict__ part_o,
                    float* __restrict__ part_ml, int n_head, int n_kv, int P, float scale, int window,
-                   int n_splits, QKPrep prep) {
+                   int n_splits, QKPrep prep, float softcap = 0.f) {
   __shared__ float s_o[4][HD / 16][4][64];
   __shared__ float s_m[4][16], s_l[4][16];
   __shared__ __attribute__((aligned(16))) bf16_t s_kv[PREP ? 2 * HD : 2];   // the row's own key, then its value
@@ -497,7 +513,8 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool
       if (r16 < n_cols)
         qf[s].u = *reinterpret_cast<const uint4*>(q + ((size_t)m_row * n_head + head) * HD + s * 32 + quad * 8);
     }
-    walk_blocks<HD>(kv, qf, b0 + wave, 4, mine, lo, p_q, p_q, scale * TI_LOG2E, edge, mx, l, o);
+    walk_blocks<HD>(kv, qf, b0 + wave, 4, mine, lo, p_q, p_q, scale * TI_LOG2E, edge, mx, l, o, NoHook{}, NoHook{},
+                    softcap * TI_LOG2E);
   }
   if (PREP && own_key && wave == 0) {
     // the row's own key and value: a block whose first key is the only one that counts
@@ -648,7 +665,7 @@ template <int HD>
 __global__ void __launch_bounds__(512)
 attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool, const int* __restrict__ table,
                     int table_stride, const int* __restrict__ tiles, const int* __restrict__ entries,
-                    bf16_t* __restrict__ out, int n_head, int n_kv, int P, float scale, int window) {
+                    bf16_t* __restrict__ out, int n_head, int n_kv, int P, float scale, int window, float softcap = 0.f) {
   const int entry = tiles[2 * blockIdx.x], first = tiles[2 * blockIdx.x + 1];
   const int row0 = entries[4 * entry], n_tok = entries[4 * entry + 1], start = entries[4 * entry + 2];
   const int head = blockIdx.y;
@@ -689,7 +706,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ poo
                                         (window <= 0 || key0 >= pos_last - window + 1) && (key0 >= tile_lo);
                     return !inside;
                   },
-                  mx, l, o);
+                  mx, l, o, NoHook{}, NoHook{}, softcap * TI_LOG2E);
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!col_ok) return;
@@ -780,7 +797,7 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                         const int* __restrict__ table, int table_stride, const int* __restrict__ tiles,
                         int n_tiles, const int* __restrict__ entries, bf16_t* __restrict__ out, int n_head,
                         int n_kv, int P, float scale, int window, float* __restrict__ part_o = nullptr,
-                        float* __restrict__ part_ml = nullptr) {
+                        float* __restrict__ part_ml = nullptr, float softcap = 0.f) {
   // gridDim.z > 1: the keys a tile sees are cut into gridDim.z runs of whole turns, workgroup z takes
   // run z and leaves its maxima, sums and unscaled outputs in part_ml [row][head][z] = (m, l) and
   // part_o [row][head][z][HD] for the kernel that merges them
@@ -1022,10 +1039,18 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     int hm = h;
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
-      float sv[16];
+      float sv[16], cv[16];
+      // a soft cap (the same in every lane) before the masks: cap tanh(s scale / cap), left in the units of the bare product
+#pragma unroll
+      for (int i = 0; i < 16; ++i) cv[i] = sc[cb][i];
+      if (softcap > 0.f) {
+        const float r = scale / softcap, back = softcap / scale;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) cv[i] = tanh_fast(cv[i] * r) * back;
+      }
       if (plain) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) sv[i] = sc[cb][i];
+        for (int i = 0; i < 16; ++i) sv[i] = cv[i];
       } else {
         asm volatile("" : "+v"(hm));
         const int hi = col_ok[cb] ? my_pos[cb] : -1;
@@ -1034,7 +1059,7 @@ attn_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
         for (int i = 0; i < 16; ++i) {
           const int key = key0 + 16 * (i >> 3) + 8 * hm + 4 * ((i >> 2) & 1) + (i & 3);
           const bool see = (key <= hi) & (key >= lo);      // bitwise on purpose: selects, no branches
-          sv[i] = see ? sc[cb][i] : -INFINITY;
+          sv[i] = see ? cv[i] : -INFINITY;
         }
       }
       float bm = sv[0];
@@ -1286,6 +1311,10 @@ static int g_decode_shared_query = 1;
 // Decode rows.  rows: which rows of the step (nullptr: rows 0..n_rows-1).  n_splits > 1 needs
 // part_o (float [n_rows, n_head, n_splits, hd]) and part_ml (float [n_rows, n_head, n_splits, 2]).
 // Returns 3 for sizes these kernels do not serve.
+// The soft cap of the call under way: the entry points whose names end in `_capped_bf16` set it around a call of
+// the plain ones, which hand it to their kernels (0: none).
+static thread_local float g_softcap = 0.f;
+
 template <bool PREP>
 static int launch_decode(const void* q, const void* pool, const int* table, int table_stride, const int* pos,
                          const int* slot, const int* rows, void* out, float* part_o, float* part_ml, int n_rows,
@@ -1306,12 +1335,12 @@ static int launch_decode(const void* q, const void* pool, const int* table, int 
     if (shared)                                                                                            \
       attn_decode_kernel<H, PREP, PREP><<<grid, 256, 0, stream>>>(                                         \
           (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, pos, slot, rows, (bf16_t*)out,        \
-          part_o, part_ml, n_head, n_kv, page_size, scale, window, n_splits, prep);                         \
+          part_o, part_ml, n_head, n_kv, page_size, scale, window, n_splits, prep, g_softcap);              \
     else                                                                                                   \
       attn_decode_kernel<H, PREP><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,   \
                                                             table_stride, pos, slot, rows, (bf16_t*)out,    \
                                                             part_o, part_ml, n_head, n_kv, page_size,       \
-                                                            scale, window, n_splits, prep);                 \
+                                                            scale, window, n_splits, prep, g_softcap);      \
     if (n_splits > 1)                                                                                       \
       attn_merge_kernel<H><<<dim3(n_rows, n_head), (H < 64 ? 64 : H), 0, stream>>>(part_o, part_ml, rows,   \
                                                                                   (bf16_t*)out, n_head,    \
@@ -1324,7 +1353,7 @@ static int launch_decode(const void* q, const void* pool, const int* table, int 
         attn_decode_kernel<32, false><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,
                                                                 table_stride, pos, slot, rows, (bf16_t*)out,
                                                                 part_o, part_ml, n_head, n_kv, page_size, scale,
-                                                                window, n_splits, prep);
+                                                                window, n_splits, prep, g_softcap);
         if (n_splits > 1)
           attn_merge_kernel<32><<<dim3(n_rows, n_head), 64, 0, stream>>>(part_o, part_ml, rows, (bf16_t*)out,
                                                                          n_head, n_splits);
@@ -1417,7 +1446,7 @@ extern "C" int ti_attention_prefill_bf16(const void* q, const void* pool, const 
   attn_prefill_lds_kernel<H, G><<<grid, 256 * G, lds, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,   \
                                                                 table_stride, tiles, n_tiles, entries,          \
                                                                 (bf16_t*)out, n_head, n_kv, page_size, scale,   \
-                                                                window)
+                                                                window, nullptr, nullptr, g_softcap)
     if (hd == 128 && groups == 2) TI_PLDS(128, 2);
     else if (hd == 128) TI_PLDS(128, 1);
     else if (groups == 2) TI_PLDS(64, 2);
@@ -1430,7 +1459,7 @@ extern "C" int ti_attention_prefill_bf16(const void* q, const void* pool, const 
   case H:                                                                                                  \
     attn_prefill_kernel<H><<<grid, 512, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table,          \
                                                      table_stride, tiles, entries, (bf16_t*)out, n_head,    \
-                                                     n_kv, page_size, scale, window);                       \
+                                                     n_kv, page_size, scale, window, g_softcap);            \
     break;
   switch (hd) {
     TI_PRE(32) TI_PRE(64) TI_PRE(128)
@@ -1483,7 +1512,7 @@ extern "C" int ti_attention_prefill_paired_bf16(const void* q, const void* pool,
 #define TI_GO(H, PAIRED)                                                                                          \
   attn_prefill_lds_kernel<H, NG, NW, ST, PAIRED, CB><<<grid, 64 * NW * NG, lds, stream>>>(                            \
       (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, n_tiles, entries, (bf16_t*)out, n_head, \
-      n_kv, page_size, scale, window, part_o, part_ml)
+      n_kv, page_size, scale, window, part_o, part_ml, g_softcap)
   if (hd == 128 && paired) TI_GO(128, true);
   else if (hd == 128) TI_GO(128, false);
   else if (paired) TI_GO(64, true);
@@ -1500,6 +1529,37 @@ extern "C" int ti_attention_prefill_paired_bf16(const void* q, const void* pool,
   }
   TI_LAUNCH_CHECK();
   return 0;
+}
+
+// The three entry points above with soft-capped scores: s <- softcap tanh(s / softcap) before the softmax.
+struct CapScope {
+  explicit CapScope(float cap) { g_softcap = cap > 0.f ? cap : 0.f; }
+  ~CapScope() { g_softcap = 0.f; }
+};
+extern "C" int ti_attention_decode_capped_bf16(const void* q, const void* pool, const int* table, int table_stride,
+                                               const int* pos, const int* slot, const int* rows, void* out, float* part_o,
+                                               float* part_ml, int n_rows, int n_head, int n_kv, int hd, int page_size,
+                                               float scale, float softcap, int window, int n_splits, hipStream_t stream) {
+  CapScope cap(softcap);
+  return ti_attention_decode_bf16(q, pool, table, table_stride, pos, slot, rows, out, part_o, part_ml, n_rows, n_head, n_kv, hd,
+                                  page_size, scale, window, n_splits, stream);
+}
+extern "C" int ti_attention_prefill_capped_bf16(const void* q, const void* pool, const int* table, int table_stride,
+                                                const int* tiles, const int* entries, void* out, int n_tiles, int n_head,
+                                                int n_kv, int hd, int page_size, float scale, float softcap, int window,
+                                                hipStream_t stream) {
+  CapScope cap(softcap);
+  return ti_attention_prefill_bf16(q, pool, table, table_stride, tiles, entries, out, n_tiles, n_head, n_kv, hd, page_size, scale,
+                                   window, stream);
+}
+extern "C" int ti_attention_prefill_paired_capped_bf16(const void* q, const void* pool, const int* table, int table_stride,
+                                                       const int* tiles, const int* entries, void* out, int n_tiles, int n_head,
+                                                       int n_kv, int hd, int page_size, float scale, float softcap, int window,
+                                                       int n_rows, float* part_o, float* part_ml, int n_splits, int paired,
+                                                       hipStream_t stream) {
+  CapScope cap(softcap);
+  return ti_attention_prefill_paired_bf16(q, pool, table, table_stride, tiles, entries, out, n_tiles, n_head, n_kv, hd, page_size,
+                                          scale, window, n_rows, part_o, part_ml, n_splits, paired, stream);
 }
 
 // ------------------------------------------------------------------- tests and measurements

@@ -159,6 +159,20 @@ int ti_attention_prefill_paired_bf16(const void* q, const void* pool, const int*
                                      int n_kv, int hd, int page_size, float scale, int window, int n_rows,
                                      float* part_o, float* part_ml, int n_splits, int paired, hipStream_t stream);
 
+// the three above with soft-capped scores: s <- softcap tanh(s / softcap) before the softmax (softcap <= 0: none)
+int ti_attention_decode_capped_bf16(const void* q, const void* pool, const int* table, int table_stride, const int* pos,
+                                    const int* slot, const int* rows, void* out, float* part_o, float* part_ml, int n_rows,
+                                    int n_head, int n_kv, int hd, int page_size, float scale, float softcap, int window,
+                                    int n_splits, hipStream_t stream);
+int ti_attention_prefill_capped_bf16(const void* q, const void* pool, const int* table, int table_stride, const int* tiles,
+                                     const int* entries, void* out, int n_tiles, int n_head, int n_kv, int hd, int page_size,
+                                     float scale, float softcap, int window, hipStream_t stream);
+int ti_attention_prefill_paired_capped_bf16(const void* q, const void* pool, const int* table, int table_stride,
+                                            const int* tiles, const int* entries, void* out, int n_tiles, int n_head,
+                                            int n_kv, int hd, int page_size, float scale, float softcap, int window,
+                                            int n_rows, float* part_o, float* part_ml, int n_splits, int paired,
+                                            hipStream_t stream);
+
 // ---- libti_sampling
 // out[r] = lowest index of the largest logit; scratch: 2 * 64 * n_rows four-byte words (two stages:
 // 64 workgroups per row, then one) or null (one workgroup reads a whole row)

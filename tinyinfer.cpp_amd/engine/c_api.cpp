@@ -1216,7 +1216,8 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
     w.slots_are_rows = n_s > 15 && s[15] != 0;
     Workspace& ws = workspace_of(&ops);
     if (op == "attention") {
-      ops.attention(w, ws, view_of(2, arg(1)), arg(0), arg(1), arg(3), (int)num(0), (int)num(1), (int)num(2), (float)num(3), (int)num(4));
+      ops.attention(w, ws, view_of(2, arg(1)), arg(0), arg(1), arg(3), (int)num(0), (int)num(1), (int)num(2), (float)num(3), (int)num(4),
+                    n_s > 16 ? (float)s[16] : 0.f);     // a soft cap of the scores
     } else {
       answer(ops.attention_from_projections(w, ws, view_of(2, arg(1)), arg(0), fptr(10), fptr(11), (float)num(13), rotation(12, 13),
                                             arg(1), num(14) != 0, arg(3), (int)num(0), (int)num(1), (int)num(2), (float)num(3),

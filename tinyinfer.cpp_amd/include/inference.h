@@ -309,8 +309,9 @@ class Ops {
                     const Tensor& q_out, int heads, int kv_heads, int head_dim);
   void attention_rows(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
                       const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window);
+  // softcap > 0: scores are capped, s <- softcap tanh(s / softcap), before the softmax
   void attention(const AttentionWork& work, Workspace& ws, const CacheView& view, const Tensor& q, const Tensor& pool,
-                 const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window);
+                 const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window, float softcap = 0.f);
   bool attention_from_projections(const AttentionWork& work, Workspace& ws, const CacheView& view, const Tensor& qkv,
                                   const float* q_w, const float* k_w, float eps, const Rotation& rot, const Tensor& pool,
                                   bool write_kv, const Tensor& out, int heads, int kv_heads, int head_dim, float scale,

@@ -296,11 +296,13 @@ class Ops:
                    g("max_context", 0), g("portion_context", 0), g("split_context", g("max_context", 0))]
         return tensors, numbers
 
-    def attention(self, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window):
-        """Attention of every row of the step over its request's pages."""
+    def attention(self, ctx, view, q, pool, out, heads, kv_heads, head_dim, scale, window, softcap: float = 0.0):
+        """Attention of every row of the step over its request's pages.  softcap > 0: scores are capped,
+        s <- softcap tanh(s / softcap), before the softmax."""
         t, n = self._work(ctx)
         libs = ["attention_generic"] + (["attention_bf16"] if q.dtype == native.torch().bfloat16 and self.use_fast_attention else [])
-        rows = [0.0, 0, 1] if getattr(ctx, "slots_are_rows", False) else []      # (unused, unused, slots[m] == m)
+        rows_are_slots = bool(getattr(ctx, "slots_are_rows", False))
+        rows = [0.0, 0, int(rows_are_slots), float(softcap)] if rows_are_slots or softcap else []   # (unused, unused, slots[m] == m, cap)
         self._call("attention", [q, pool, view.table, out] + t, [heads, kv_heads, head_dim, scale, int(window or 0)] + n + rows,
                    fold=(1,), libs=libs)
 

@@ -790,7 +790,7 @@ bool Ops::attention_from_projections(const AttentionWork& work, Workspace& ws, c
 }
 
 void Ops::attention(const AttentionWork& work, Workspace& ws, const CacheView& view, const Tensor& q, const Tensor& pool,
-                    const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window) {
+                    const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window, float softcap) {
   TunedScope tuned(*this, "attention_bf16");
   TIMED("attention rows=" + std::to_string(work.M) + (work.decode_only ? " decode" : " tiles=" + std::to_string(work.n_tiles) + " single=" + std::to_string(work.n_decode_rows)) + " context<=" + std::to_string(work.max_context));
   bool done = false;
@@ -817,16 +817,16 @@ void Ops::attention(const AttentionWork& work, Workspace& ws, const CacheView& v
           part_o = (float*)ws.get("attn.portion_o", (size_t)work.M * heads * S * head_dim * 4);
           part_ml = (float*)ws.get("attn.portion_ml", (size_t)work.M * heads * S * 2 * 4);
         }
-        int rc = KERNEL("attention_bf16", ti_attention_prefill_paired_bf16)(
+        int rc = KERNEL("attention_bf16", ti_attention_prefill_paired_capped_bf16)(
             q.data, pool.data, view.table, view.table_width, work.tiles_small, work.entry_meta, out.data, work.n_tiles_small,
-            heads, kv_heads, head_dim, P, scale, window, (int)work.M, part_o, part_ml, S, paired ? 1 : 0,
+            heads, kv_heads, head_dim, P, scale, softcap, window, (int)work.M, part_o, part_ml, S, paired ? 1 : 0,
             (hipStream_t)stream);
         if (rc == 3) done = false;
         else check("attention_bf16", rc, "attention(prefill, paired)");
       } else if (work.n_tiles) {
-        int rc = KERNEL("attention_bf16", ti_attention_prefill_bf16)(
+        int rc = KERNEL("attention_bf16", ti_attention_prefill_capped_bf16)(
             q.data, pool.data, view.table, view.table_width, work.tiles, work.entry_meta, out.data, work.n_tiles, heads,
-            kv_heads, head_dim, P, scale, window, (hipStream_t)stream);
+            kv_heads, head_dim, P, scale, softcap, window, (hipStream_t)stream);
         if (rc == 3) done = false;
         else check("attention_bf16", rc, "attention(prefill)");
       }
@@ -840,17 +840,19 @@ void Ops::attention(const AttentionWork& work, Workspace& ws, const CacheView& v
           part_o = (float*)ws.get("attn.part_o", (size_t)n_dec * heads * S * head_dim * 4);
           part_ml = (float*)ws.get("attn.part_ml", (size_t)n_dec * heads * S * 2 * 4);
         }
-        int rc = KERNEL("attention_bf16", ti_attention_decode_bf16)(
+        int rc = KERNEL("attention_bf16", ti_attention_decode_capped_bf16)(
             q.data, pool.data, view.table, view.table_width, work.positions,
             (work.slots_are_rows && !rows && view.table_width <= 1024 && use.early_page_ids) ? nullptr : work.slots, rows, out.data,
-            part_o, part_ml, n_dec, heads, kv_heads, head_dim, P, scale, window, S, (hipStream_t)stream);
+            part_o, part_ml, n_dec, heads, kv_heads, head_dim, P, scale, softcap, window, S, (hipStream_t)stream);
         if (rc == 3) done = false;
         else check("attention_bf16", rc, "attention(decode)");
       }
     }
   }
   took(done ? "[mfma]" : "[generic]");
-  if (!done)
+  if (!done && softcap > 0.f)
+    attention_capped(q, pool, view, work.positions, work.slots, out, heads, kv_heads, head_dim, head_dim, scale, softcap, window);
+  else if (!done)
     attention_rows(q, pool, view, work.positions, work.slots, out, heads, kv_heads, head_dim, scale, window);
 }
 

@@ -656,7 +656,10 @@ class Attention final : public MixerPart {
     Tensor q = ctx.buf("attn.q", ctx.act_dtype, {M, nq});
     ctx.ops.qkv_split_write(qkv, ctx.positions, ctx.slots, view, pool, q, heads, kv_heads, head_dim, v_dim, temp_coef, temp_every);
     Tensor a = ctx.buf("attn.out", ctx.act_dtype, {M, no});
-    ctx.ops.attention_capped(q, pool, view, ctx.positions, ctx.slots, a, heads, kv_heads, head_dim, v_dim, scale, softcap, window);
+    if (v_dim == head_dim)      // the step's tiles through the matrix cores where they serve the size, else row by row
+      ctx.ops.attention(work(ctx), ctx.ws, view, q, pool, a, heads, kv_heads, head_dim, scale, window, softcap);
+    else
+      ctx.ops.attention_capped(q, pool, view, ctx.positions, ctx.slots, a, heads, kv_heads, head_dim, v_dim, scale, softcap, window);
     ctx.ops.linear(a, w_o, out, epi, epi == Ops::Add);
   }
   void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override {
@@ -784,6 +787,7 @@ class DenseFFN final : public FeedForwardPart {
     n_act = tensor_name(p, "act", prefix, "act");
   }
   const char* kind_name() const override { return "dense"; }
+  bool takes_lazy_norm() const override { return true; }       // h goes into the up product and nowhere else
   bool reads_through_ops() const override { return true; }
   bool can_store() const override { return true; }
   std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
@@ -848,6 +852,7 @@ class MLSTM final : public MixerPart {
     width = 2 * nq + 2 * nv + 2 * heads;
   }
   const char* kind_name() const override { return "mlstm"; }
+  bool takes_lazy_norm() const override { return true; }       // h goes into the stacked projection and nowhere else
   bool reads_through_ops() const override { return true; }
   bool can_store() const override { return true; }
   std::string name(const char* t) const { return join(prefix, t); }
@@ -975,7 +980,10 @@ class ParallelBlock final : public BlockPart {
   }
   void forward(StepContext& ctx, const Tensor& x) override {
     if (!norm1->reads_through_ops()) ctx.ops.flush();
-    const Rows h = norm1->forward(ctx, x, nullptr, 0, false);
+    // each branch feeds h to one product: where a product can take the norm in (a step of few rows), the rows stay
+    // uncomputed and each branch's first product norms them itself; the first product that cannot computes them for all
+    bool lazy = norm1->can_be_lazy() && mixer->takes_lazy_norm() && (!ffn || ffn->takes_lazy_norm());
+    const Rows h = norm1->forward(ctx, x, nullptr, 0, lazy);
     const int64_t M = x.shape[0];
     Tensor y1 = ctx.buf("parallel.y1", DType::F32, {M, dim});
     if (!mixer->reads_through_ops()) ctx.ops.flush();
