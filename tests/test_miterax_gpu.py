@@ -67,13 +67,14 @@ def test_add_sinusoid_and_add_row(ops):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_xielu(ops, dtype):
     rng = np.random.default_rng(3)
-    z = np.concatenate([rng.normal(size=500) * 3, [0.0, -1e-4, 1e-4, -20.0, 15.0]]).astype(np.float32)
-    for p, q in [(0.3, -0.7), (-2.0, 1.5), (0.0, 0.0)]:
-        out = torch.empty(len(z), device="cuda", dtype=DT[dtype])
-        ops.xielu(dev(z), dev([p, q]), out)
-        want = plain.xielu(z.astype(np.float64), p, q)
-        tol = 2e-6 * (1 + np.abs(want)) if dtype == "float32" else 2.0 ** -8 * np.abs(want) + 1e-6
-        assert (np.abs(f64(out) - want) <= tol).all()
+    for n in (500, 507):            # with the five below: a count that is no multiple of eight, and one that is
+        z = np.concatenate([rng.normal(size=n) * 3, [0.0, -1e-4, 1e-4, -20.0, 15.0]]).astype(np.float32)
+        for p, q in [(0.3, -0.7), (-2.0, 1.5), (0.0, 0.0)]:
+            out = torch.empty(len(z), device="cuda", dtype=DT[dtype])
+            ops.xielu(dev(z), dev([p, q]), out)
+            want = plain.xielu(z.astype(np.float64), p, q)
+            tol = 2e-6 * (1 + np.abs(want)) if dtype == "float32" else 2.0 ** -8 * np.abs(want) + 1e-6
+            assert (np.abs(f64(out) - want) <= tol).all()
 
 
 def test_scaled_add(ops):
@@ -262,6 +263,61 @@ def test_mlstm_scan_carries_its_state(ops, heads, dk, dv):
     assert float(state[1].abs().max()) == 0.0                  # a slot nobody used stays untouched
 
 
+@pytest.mark.parametrize("heads,dk,dv,chunk", [(2, 16, 24, 64), (1, 130, 70, 64), (2, 64, 64, 16), (1, 128, 128, 64)])
+def test_mlstm_scan_in_chunks(ops, heads, dk, dv, chunk):
+    """Entries of 300, 1, 64, 65 and 200 tokens on states that an earlier step left, their tokens cut into chunks that run
+    side by side: the outputs and the states against the recurrence token by token."""
+    rng = np.random.default_rng(dk * 7 + dv)
+    cap = 6.0
+    N = heads * (2 * dk + 2 * dv + 2)
+    cols = dict(q=0, k=heads * dk, v=2 * heads * dk, i=2 * heads * dk + 2 * heads * dv, f=2 * heads * dk + 2 * heads * dv + heads)
+    per_head = dk * dv + dk + 1
+    state = torch.zeros(6, heads, per_head, device="cuda")
+    bi, bf = rng.normal(size=heads), rng.normal(size=heads) + 2.0
+    ref = {}
+
+    def step(lengths, slots, chunked):
+        M = sum(lengths)
+        proj = rng.normal(size=(M, N)).astype(np.float32)
+        proj[:, cols["i"]:cols["i"] + heads] *= 3.0
+        entries, chunks, spans, row = [], [], [], 0
+        for e, (n_tok, s) in enumerate(zip(lengths, slots)):
+            entries.append([row, n_tok, 0, s])
+            n = -(-n_tok // chunk)
+            spans.append([len(chunks), n])
+            for k in range(n):
+                chunks.append([e, row + k * chunk, min(chunk, n_tok - k * chunk), (1 if k == 0 else 0) | (2 if k == n - 1 else 0)])
+            row += n_tok
+        o = torch.full((M, heads * dv), 7.0, device="cuda")
+        more = dict(chunks=dev(chunks, torch.int32), spans=dev(spans, torch.int32)) if chunked else {}
+        ops.mlstm_scan(dev(proj), dev(bi), dev(bf), state, dev(entries, torch.int32), o, heads, dk, dv, cap, dk ** -0.5,
+                       (cols["q"], cols["k"], cols["v"], cols["i"], cols["f"]), **more)
+        p = proj.astype(np.float64)
+        want = np.zeros((M, heads, dv))
+        for (row0, n_tok, _, s) in entries:
+            for h in range(heads):
+                S, n, m = ref.get((s, h), (np.zeros((dk, dv)), np.zeros(dk), 0.0))
+                rows = slice(row0, row0 + n_tok)
+                q = p[rows, cols["q"] + h * dk: cols["q"] + (h + 1) * dk] * np.float64(np.float32(dk ** -0.5))
+                k = p[rows, cols["k"] + h * dk: cols["k"] + (h + 1) * dk]
+                v = p[rows, cols["v"] + h * dv: cols["v"] + (h + 1) * dv]
+                ig = cap * np.tanh((p[rows, cols["i"] + h] + bi[h]) / cap)
+                fg = plain.logsigmoid(cap * np.tanh((p[rows, cols["f"] + h] + bf[h]) / cap))
+                want[rows, h], S, n, m = plain_cell(q, k, v, ig, fg, S, n, m)
+                ref[(s, h)] = (S, n, m)
+        got = f64(o).reshape(M, heads, dv)
+        assert np.abs(got - want).max() < 3e-4 * max(1.0, np.abs(want).max())
+
+    step([5, 20, 3], [4, 0, 2], chunked=False)
+    step([300, 1, 64, 65, 200], [4, 1, 0, 3, 2], chunked=True)
+    step([1, 1, 130], [4, 3, 5], chunked=True)
+    st = f64(state)
+    for (s, h), (S, n, m) in ref.items():
+        assert np.abs(st[s, h, : dk * dv].reshape(dk, dv) - S).max() < 3e-4 * max(1.0, np.abs(S).max())
+        assert np.abs(st[s, h, dk * dv: dk * dv + dk] - n).max() < 3e-4 * max(1.0, np.abs(n).max())
+        assert abs(st[s, h, -1] - m) < 1e-4
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_gated_head_norm(ops, dtype):
     rng = np.random.default_rng(8)
@@ -395,6 +451,31 @@ def test_a_state_slot_used_again_starts_from_zero(folders):
         got = replay(engine, traces.portions({r: requests[r]}))
         w, where = worst(got, {r: want[r]})
         assert w < TOL["float32"], (r, w, where)
+
+
+def test_long_portions_beside_single_tokens(folders):
+    """Steps that hold a portion of hundreds of tokens (the recurrent layers cut it into chunks that run side by side)
+    beside other requests' single tokens and short portions, in 32-bit and in bfloat16."""
+    from tinyinfer_amd.engine import StepEntry
+    for name in ("loop3", "odd"):
+        folder, _, _, w = folders(name)
+        config = mm.CONFIGS[name]
+        toks = {r: random_tokens(n, config["vocab"], 50 + i) for i, (r, n) in enumerate({"p": 520, "q": 40, "r": 260}.items())}
+        want = {r: plain.forward(config, w, t) for r, t in toks.items()}
+        steps = [[("q", 0, 30)], [("p", 0, 300), ("q", 30, 1)], [("p", 300, 193), ("q", 31, 1), ("r", 0, 7)],
+                 [("r", 7, 253), ("p", 493, 27), ("q", 32, 8)]]
+        for dtype in ("float32", "bfloat16"):
+            engine = build_engine(folder, dtype, 1024)
+            got = {r: [] for r in toks}
+            for step in steps:
+                logits = engine.step([StepEntry(r, toks[r][lo:lo + n], list(range(n))) for r, lo, n in step]).cpu().numpy().astype(np.float64)
+                i = 0
+                for r, lo, n in step:
+                    got[r].append(logits[i:i + n])
+                    i += n
+                engine.cache.check()
+            ok, seen = within({r: np.concatenate(v) for r, v in got.items()}, want, dtype)
+            assert ok, (name, dtype, seen)
 
 
 def test_long_context_and_long_decoding(folders):

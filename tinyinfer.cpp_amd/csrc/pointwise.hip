@@ -60,13 +60,51 @@ __global__ void xielu_kernel(const float* __restrict__ z, const float* __restric
     st<T>(out + i, xielu_f(z[i], ap, an));
 }
 
+// The same, eight elements a thread (n a multiple of 8, 16-byte aligned operands).  Rounded to bfloat16 the
+// result keeps 8 bits, so exp(z) - 1 from the hardware's exponential (absolute error 1e-7) serves there;
+// 32-bit output keeps expm1.
+template <typename T>
+__global__ void __launch_bounds__(256)
+xielu_wide_kernel(const float* __restrict__ z, const float* __restrict__ act, T* __restrict__ out, long n8) {
+  const float ap = softplus_f(act[0]), an = 0.5f + softplus_f(act[1]);
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += (long)gridDim.x * blockDim.x) {
+    const float4 a = reinterpret_cast<const float4*>(z)[2 * i], b = reinterpret_cast<const float4*>(z)[2 * i + 1];
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    float y[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      if (sizeof(T) == 2) {
+        const float e = __builtin_amdgcn_exp2f(fminf(v[k], 0.f) * 1.4426950408889634f) - 1.0f;
+        y[k] = v[k] > 0.f ? fmaf(ap * v[k], v[k], 0.5f * v[k]) : fmaf(an, e - v[k], 0.5f * v[k]);
+      } else {
+        y[k] = xielu_f(v[k], ap, an);
+      }
+    }
+    if (sizeof(T) == 2) {
+      reinterpret_cast<uint4*>(out)[i] = make_uint4(pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3]), pack_bf16x2(y[4], y[5]),
+                                                    pack_bf16x2(y[6], y[7]));
+    } else {
+      reinterpret_cast<float4*>(out)[2 * i] = make_float4(y[0], y[1], y[2], y[3]);
+      reinterpret_cast<float4*>(out)[2 * i + 1] = make_float4(y[4], y[5], y[6], y[7]);
+    }
+  }
+}
+
 extern "C" int ti_xielu(int out_dtype, const float* z, const float* act, void* out, long n, hipStream_t stream) {
   TI_REQUIRE(n >= 0, "xielu: bad count %ld", n);
   if (n == 0) return 0;
+  TI_REQUIRE(out_dtype == TI_F32 || out_dtype == TI_BF16, "xielu: unknown dtype %d", out_dtype);
+  if (n % 8 == 0 && (((uintptr_t)z | (uintptr_t)out) & 15) == 0) {
+    const long n8 = n / 8;
+    const unsigned blocks = (unsigned)((n8 + 255) / 256 < 8192 ? (n8 + 255) / 256 : 8192);
+    if (out_dtype == TI_F32) xielu_wide_kernel<float><<<blocks, 256, 0, stream>>>(z, act, (float*)out, n8);
+    else xielu_wide_kernel<bf16_t><<<blocks, 256, 0, stream>>>(z, act, (bf16_t*)out, n8);
+    TI_LAUNCH_CHECK();
+    return 0;
+  }
   const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
   if (out_dtype == TI_F32) xielu_kernel<float><<<blocks, 256, 0, stream>>>(z, act, (float*)out, n);
-  else if (out_dtype == TI_BF16) xielu_kernel<bf16_t><<<blocks, 256, 0, stream>>>(z, act, (bf16_t*)out, n);
-  else TI_REQUIRE(false, "xielu: unknown dtype %d", out_dtype);
+  else xielu_kernel<bf16_t><<<blocks, 256, 0, stream>>>(z, act, (bf16_t*)out, n);
   TI_LAUNCH_CHECK();
   return 0;
 }
@@ -83,11 +121,40 @@ __global__ void scaled_add_kernel(float* __restrict__ x, const float* __restrict
   }
 }
 
+// the same, four channels a thread (H a multiple of 4, 16-byte aligned operands): the same arithmetic, the same bits
+__global__ void __launch_bounds__(256)
+scaled_add_wide_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ sa,
+                       const float* __restrict__ b, const float* __restrict__ sb, long n4, int H4) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (long)gridDim.x * blockDim.x) {
+    const int c = (int)(i % H4);
+    const float4 one = make_float4(1.f, 1.f, 1.f, 1.f);
+    const float4 av = reinterpret_cast<const float4*>(a)[i], s1 = sa ? reinterpret_cast<const float4*>(sa)[c] : one;
+    float4 y = make_float4(av.x * s1.x, av.y * s1.y, av.z * s1.z, av.w * s1.w);
+    if (b) {
+      const float4 bv = reinterpret_cast<const float4*>(b)[i], s2 = sb ? reinterpret_cast<const float4*>(sb)[c] : one;
+      y = make_float4(fmaf(bv.x, s2.x, y.x), fmaf(bv.y, s2.y, y.y), fmaf(bv.z, s2.z, y.z), fmaf(bv.w, s2.w, y.w));
+    }
+    float4 xv = reinterpret_cast<float4*>(x)[i];
+    xv.x += y.x;
+    xv.y += y.y;
+    xv.z += y.z;
+    xv.w += y.w;
+    reinterpret_cast<float4*>(x)[i] = xv;
+  }
+}
+
 extern "C" int ti_scaled_add(float* x, const float* a, const float* sa, const float* b, const float* sb, int M, int H,
                              hipStream_t stream) {
   TI_REQUIRE(M >= 0 && H > 0 && a, "scaled_add: bad sizes M=%d H=%d", M, H);
   if (M == 0) return 0;
   const long n = (long)M * H;
+  if (H % 4 == 0 && (((uintptr_t)x | (uintptr_t)a | (uintptr_t)sa | (uintptr_t)b | (uintptr_t)sb) & 15) == 0) {
+    const long n4 = n / 4;
+    const unsigned wide = (unsigned)((n4 + 255) / 256 < 8192 ? (n4 + 255) / 256 : 8192);
+    scaled_add_wide_kernel<<<wide, 256, 0, stream>>>(x, a, sa, b, sb, n4, H / 4);
+    TI_LAUNCH_CHECK();
+    return 0;
+  }
   const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
   scaled_add_kernel<<<blocks, 256, 0, stream>>>(x, a, sa, b, sb, n, H);
   TI_LAUNCH_CHECK();
@@ -108,14 +175,37 @@ __global__ void qkv_split_write_kernel(const float* __restrict__ qkv, const int*
   const int nq = n_head * dk, nk = n_kv * dk, nv = n_kv * dv;
   const float* row = qkv + (size_t)m * (nq + nk + nv);
   const float temp = (coef != 0.f && every > 0) ? 1.f + coef * logf((float)((p + 1) / every) + 1.f) : 1.f;
-  for (int e = threadIdx.x; e < nq; e += blockDim.x) st<T>(q_out + (size_t)m * nq + e, row[e] * temp);
+  // four elements a thread where every run of them is aligned (the products are the same, so are the bits)
+  const bool wide = (dk % 4 == 0) && (dv % 4 == 0) && (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)pool) & 15) == 0;
   const int page = table[(size_t)slot[m] * table_stride + p / P];
-  if (page < 0) return;   // the host reserves pages first; never write astray
   const int r = p % P;
-  T* base = pool + (size_t)page * ((size_t)n_kv * P * (dk + dv));
-  for (int e = threadIdx.x; e < nk; e += blockDim.x) {
-    const int h = e / dk, d = e % dk;
-    st<T>(base + ((size_t)h * P + r) * dk + d, row[nq + e]);
+  T* base = pool + (size_t)max(page, 0) * ((size_t)n_kv * P * (dk + dv));
+  if (wide) {
+    for (int e = threadIdx.x * 4; e < nq; e += blockDim.x * 4) {
+      const float4 v = *reinterpret_cast<const float4*>(row + e);
+      T* dst = q_out + (size_t)m * nq + e;
+      st<T>(dst, v.x * temp);
+      st<T>(dst + 1, v.y * temp);
+      st<T>(dst + 2, v.z * temp);
+      st<T>(dst + 3, v.w * temp);
+    }
+    if (page < 0) return;   // the host reserves pages first; never write astray
+    for (int e = threadIdx.x * 4; e < nk; e += blockDim.x * 4) {
+      const int h = e / dk, d = e % dk;
+      const float4 v = *reinterpret_cast<const float4*>(row + nq + e);
+      T* dst = base + ((size_t)h * P + r) * dk + d;
+      st<T>(dst, v.x);
+      st<T>(dst + 1, v.y);
+      st<T>(dst + 2, v.z);
+      st<T>(dst + 3, v.w);
+    }
+  } else {
+    for (int e = threadIdx.x; e < nq; e += blockDim.x) st<T>(q_out + (size_t)m * nq + e, row[e] * temp);
+    if (page < 0) return;
+    for (int e = threadIdx.x; e < nk; e += blockDim.x) {
+      const int h = e / dk, d = e % dk;
+      st<T>(base + ((size_t)h * P + r) * dk + d, row[nq + e]);
+    }
   }
   T* vbase = base + (size_t)n_kv * P * dk;
   for (int e = threadIdx.x; e < nv; e += blockDim.x) {

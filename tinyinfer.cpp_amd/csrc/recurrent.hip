@@ -25,12 +25,21 @@ TI_ERROR_API
 
 __device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
-template <int RPL, int MAXT>
+// MODE 0: each workgroup one (entry, head): from the request's state slot over all its tokens and back into the slot.
+// Long portions are cut into chunks (`chunks` int32 [n][4] = (entry, first row, tokens, 1 if the entry's first chunk +
+// 2 if its last)), three launches:
+// MODE 1: every chunk but an entry's last from an empty memory (S = 0, n = 0, m = -inf), no output: what the chunk
+//         alone adds (S, n, its maximum m and F, the sum of its log forget gates) goes to `chunk_buf`;
+//         then mlstm_combine_kernel walks an entry's chunks and leaves in `chunk_buf` the state each chunk starts from;
+// MODE 2: every chunk from that state (an entry of a single chunk: from its slot) with output; an entry's last chunk
+//         writes the slot.
+// chunk_buf per (chunk, head): S [dk][dv], n [dk], m of the chunk alone, F, m the chunk starts from.
+template <int RPL, int MAXT, int MODE>
 __global__ void __launch_bounds__(MAXT)
 mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, int off_v, int off_i, int off_f,
                   const float* __restrict__ bias_i, const float* __restrict__ bias_f, float* __restrict__ state,
-                  long slot_stride, const int* __restrict__ entries, float* __restrict__ o, int heads, int dk, int dv,
-                  float cap, float q_scale) {
+                  long slot_stride, const int* __restrict__ entries, const int* __restrict__ chunks,
+                  float* __restrict__ chunk_buf, float* __restrict__ o, int heads, int dk, int dv, float cap, float q_scale) {
   constexpr int DP = RPL * ML_RG;   // rows, padded
   extern __shared__ __align__(16) float lds[];
   float* lq = lds;                        // [ML_TB][DP]
@@ -38,27 +47,45 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, 
   float* lv = lk + ML_TB * DP;            // [ML_TB][dv]
   float* lgi = lv + ML_TB * dv;           // [ML_TB]
   float* lgf = lgi + ML_TB;               // [ML_TB]
-  const int e = blockIdx.x, h = blockIdx.y;
-  const int row0 = entries[4 * e], n_tok = entries[4 * e + 1], slot = entries[4 * e + 3];
+  const int unit = blockIdx.x, h = blockIdx.y;
+  int e = unit, row0, n_tok, flags = 3;
+  if (MODE == 0) {
+    row0 = entries[4 * e];
+    n_tok = entries[4 * e + 1];
+  } else {
+    e = chunks[4 * unit];
+    row0 = chunks[4 * unit + 1];
+    n_tok = chunks[4 * unit + 2];
+    flags = chunks[4 * unit + 3];
+  }
+  const bool whole = (flags & 3) == 3, last = (flags & 2) != 0;
+  if (MODE == 1 && last) return;          // nobody reads what an entry's last chunk adds alone
+  const int slot = entries[4 * e + 3];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, rg = lane >> 4, c = lane & 15;
   const int n_waves = blockDim.x >> 6;
-  float* S_base = state + (size_t)slot * slot_stride + (size_t)h * ((size_t)dk * dv + dk + 1);
-  float* n_base = S_base + (size_t)dk * dv;
-  float* m_ptr = n_base + dk;
+  const size_t per_head = (size_t)dk * dv + dk + 1;
+  float* slot_base = state + (size_t)slot * slot_stride + (size_t)h * per_head;
+  float* cb = (MODE == 0) ? nullptr : chunk_buf + ((size_t)unit * heads + h) * (per_head + 2);
+  // where the memory comes from and where it goes
+  const bool from_slot = MODE == 0 || (MODE == 2 && whole);
+  const float* S_src = from_slot ? slot_base : cb;
+  const float* m_src = from_slot ? slot_base + per_head - 1 : cb + per_head + 1;
+  float* S_dst = (MODE == 0 || (MODE == 2 && last)) ? slot_base : (MODE == 1 ? cb : nullptr);
   const int ov = heads * dv;
   const int span = n_waves * ML_COLS;
   float S[RPL], nn[RPL];
-  float m = 0.f;
+  float m = 0.f, F = 0.f;
   for (int j0 = 0; j0 < dv; j0 += span) {
     const int j = j0 + wave * ML_COLS + c;
     const bool active = j < dv;
 #pragma unroll
     for (int i = 0; i < RPL; ++i) {
       const int r = rg * RPL + i;
-      S[i] = (active && r < dk) ? S_base[(size_t)r * dv + j] : 0.f;
-      nn[i] = r < dk ? n_base[r] : 0.f;
+      S[i] = (MODE != 1 && active && r < dk) ? S_src[(size_t)r * dv + j] : 0.f;
+      nn[i] = (MODE != 1 && r < dk) ? S_src[(size_t)dk * dv + r] : 0.f;
     }
-    m = *m_ptr;
+    m = (MODE == 1) ? -INFINITY : *m_src;
+    F = 0.f;
     for (int t0 = 0; t0 < n_tok; t0 += ML_TB) {
       const int tb = n_tok - t0 < ML_TB ? n_tok - t0 : ML_TB;
       __syncthreads();   // the reads of the tokens before are over
@@ -84,6 +111,7 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, 
         const float m_new = fmaxf(fg + m, ig);
         const float decay = expf(fg + m - m_new), take = expf(ig - m_new);
         m = m_new;
+        F += fg;
         const float tv = active ? take * lv[t * dv + j] : 0.f;
         const float4* q4 = reinterpret_cast<const float4*>(lq + t * DP + rg * RPL);
         const float4* k4 = reinterpret_cast<const float4*>(lk + t * DP + rg * RPL);
@@ -96,37 +124,112 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, 
           for (int u = 0; u < 4; ++u) {
             S[i + u] = fmaf(ka[u], tv, decay * S[i + u]);
             nn[i + u] = fmaf(take, ka[u], decay * nn[i + u]);
-            acc = fmaf(S[i + u], qa[u], acc);
-            nq = fmaf(nn[i + u], qa[u], nq);
+            if (MODE != 1) {
+              acc = fmaf(S[i + u], qa[u], acc);
+              nq = fmaf(nn[i + u], qa[u], nq);
+            }
           }
         }
-        acc += __shfl_xor(acc, 16, TI_WAVE);
-        acc += __shfl_xor(acc, 32, TI_WAVE);
-        nq += __shfl_xor(nq, 16, TI_WAVE);
-        nq += __shfl_xor(nq, 32, TI_WAVE);
-        const float denom = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
-        if (rg == 0 && active) o[(size_t)(row0 + t0 + t) * ov + h * dv + j] = acc / denom;
+        if (MODE != 1) {
+          acc += __shfl_xor(acc, 16, TI_WAVE);
+          acc += __shfl_xor(acc, 32, TI_WAVE);
+          nq += __shfl_xor(nq, 16, TI_WAVE);
+          nq += __shfl_xor(nq, 32, TI_WAVE);
+          const float denom = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
+          if (rg == 0 && active) o[(size_t)(row0 + t0 + t) * ov + h * dv + j] = acc / denom;
+        }
       }
     }
-    if (active) {
+    if (active && S_dst) {
 #pragma unroll
       for (int i = 0; i < RPL; ++i) {
         const int r = rg * RPL + i;
-        if (r < dk) S_base[(size_t)r * dv + j] = S[i];
+        if (r < dk) S_dst[(size_t)r * dv + j] = S[i];
       }
     }
   }
   // n and m: every lane holds the same; one lane per quarter of the rows writes, after all have read
   __syncthreads();
-  if (wave == 0 && c == 0) {
+  if (S_dst && wave == 0 && c == 0) {
 #pragma unroll
     for (int i = 0; i < RPL; ++i) {
       const int r = rg * RPL + i;
-      if (r < dk) n_base[r] = nn[i];
+      if (r < dk) S_dst[(size_t)dk * dv + r] = nn[i];
     }
-    if (rg == 0) *m_ptr = m;
+    if (rg == 0) {
+      S_dst[per_head - 1] = m;
+      if (MODE == 1) S_dst[per_head] = F;
+    }
   }
 }
+
+// An entry's chunks in order, for every entry of more than one chunk (`spans` int32 [R][2] = (first chunk, chunks)):
+// with the running state (S, n, m) starting at the request's slot, chunk c gets the state it starts from in place
+// of what it added alone (A_c, a_c, m_c, F_c), and the running state goes on as
+//   m' = max(F_c + m, m_c);  S' = exp(F_c + m - m') S + exp(m_c - m') A_c;  n' likewise
+// (the recurrence of the cell, taken a chunk at a time).  grid (entries, heads, slices of the elements).
+__global__ void __launch_bounds__(256)
+mlstm_combine_kernel(const float* __restrict__ state, long slot_stride, const int* __restrict__ entries,
+                     const int* __restrict__ spans, float* __restrict__ chunk_buf, int heads, int dk, int dv) {
+  const int e = blockIdx.x, h = blockIdx.y;
+  const int first = spans[2 * e], n = spans[2 * e + 1];
+  if (n < 2) return;
+  const size_t per_head = (size_t)dk * dv + dk + 1, elems = per_head - 1, stride = per_head + 2;
+  const float* slot_base = state + (size_t)entries[4 * e + 3] * slot_stride + (size_t)h * per_head;
+  float m = slot_base[per_head - 1];
+  constexpr int PER = 8;            // elements a thread carries through the chunks
+  const size_t base = ((size_t)blockIdx.z * blockDim.x + threadIdx.x) * PER;
+  float run[PER];
+#pragma unroll
+  for (int k = 0; k < PER; ++k) run[k] = base + k < elems ? slot_base[base + k] : 0.f;
+  for (int cidx = 0; cidx < n; ++cidx) {
+    float* cb = chunk_buf + ((size_t)(first + cidx) * heads + h) * stride;
+    const float m_c = cb[per_head - 1], F_c = cb[per_head];
+    float loc[PER];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) loc[k] = (cidx + 1 < n && base + k < elems) ? cb[base + k] : 0.f;
+#pragma unroll
+    for (int k = 0; k < PER; ++k)
+      if (base + k < elems) cb[base + k] = run[k];
+    if (blockIdx.z == 0 && threadIdx.x == 0) cb[per_head + 1] = m;
+    if (cidx + 1 < n) {
+      const float m_new = fmaxf(F_c + m, m_c);
+      const float a = expf(F_c + m - m_new), b = expf(m_c - m_new);
+#pragma unroll
+      for (int k = 0; k < PER; ++k) run[k] = fmaf(b, loc[k], a * run[k]);
+      m = m_new;
+    }
+  }
+}
+
+static int mlstm_shape(int heads, int dk, int dv, float cap, int* rpl, int* waves, size_t* lds) {
+  TI_REQUIRE(heads > 0 && heads <= 65535 && dk >= 1 && dk <= 256 && dv >= 1, "mlstm: heads %d, key size %d (up to 256), value size %d",
+             heads, dk, dv);
+  TI_REQUIRE(cap > 0.f, "mlstm: the gates' cap must be positive");
+  *rpl = dk <= 32 ? 8 : dk <= 64 ? 16 : dk <= 128 ? 32 : 64;
+  const int max_waves = *rpl <= 16 ? 16 : *rpl == 32 ? 8 : 4;
+  *waves = (dv + ML_COLS - 1) / ML_COLS;
+  if (*waves > max_waves) *waves = max_waves;
+  *lds = ((size_t)ML_TB * (2 * *rpl * ML_RG + dv) + 2 * ML_TB) * sizeof(float);
+  TI_REQUIRE(*lds <= 64 * 1024, "mlstm: value size %d needs %zu bytes of LDS", dv, *lds);
+  return 0;
+}
+
+#define ML_LAUNCH(MODE, GRID)                                                                                          \
+  do {                                                                                                                 \
+    if (rpl == 8)                                                                                                      \
+      mlstm_scan_kernel<8, 1024, MODE><<<GRID, waves * 64, lds, stream>>>(proj, ld, off_q, off_k, off_v, off_i, off_f, bias_i, \
+          bias_f, state, slot_stride, entries, chunks, chunk_buf, o, heads, dk, dv, cap, q_scale);                     \
+    else if (rpl == 16)                                                                                                \
+      mlstm_scan_kernel<16, 1024, MODE><<<GRID, waves * 64, lds, stream>>>(proj, ld, off_q, off_k, off_v, off_i, off_f, bias_i, \
+          bias_f, state, slot_stride, entries, chunks, chunk_buf, o, heads, dk, dv, cap, q_scale);                     \
+    else if (rpl == 32)                                                                                                \
+      mlstm_scan_kernel<32, 512, MODE><<<GRID, waves * 64, lds, stream>>>(proj, ld, off_q, off_k, off_v, off_i, off_f, bias_i, \
+          bias_f, state, slot_stride, entries, chunks, chunk_buf, o, heads, dk, dv, cap, q_scale);                     \
+    else                                                                                                               \
+      mlstm_scan_kernel<64, 256, MODE><<<GRID, waves * 64, lds, stream>>>(proj, ld, off_q, off_k, off_v, off_i, off_f, bias_i, \
+          bias_f, state, slot_stride, entries, chunks, chunk_buf, o, heads, dk, dv, cap, q_scale);                     \
+  } while (0)
 
 // proj f32 [M, ld]: the projections of the step's rows; off_*: the columns where the heads' q [heads][dk],
 // k [heads][dk], v [heads][dv] and the gate pre-activations i, f [heads] start.  state f32: per slot
@@ -136,25 +239,40 @@ extern "C" int ti_mlstm_scan(const float* proj, int ld, int off_q, int off_k, in
                              const float* bias_i, const float* bias_f, float* state, long slot_stride, const int* entries,
                              int n_entries, float* o, int heads, int dk, int dv, float cap, float q_scale,
                              hipStream_t stream) {
-  TI_REQUIRE(heads > 0 && heads <= 65535 && dk >= 1 && dk <= 256 && dv >= 1, "mlstm: heads %d, key size %d (up to 256), value size %d",
-             heads, dk, dv);
-  TI_REQUIRE(cap > 0.f, "mlstm: the gates' cap must be positive");
+  int rpl, waves;
+  size_t lds;
+  if (int rc = mlstm_shape(heads, dk, dv, cap, &rpl, &waves, &lds)) return rc;
   if (n_entries == 0) return 0;
-  const int rpl = dk <= 32 ? 8 : dk <= 64 ? 16 : dk <= 128 ? 32 : 64;
-  const int max_waves = rpl <= 16 ? 16 : rpl == 32 ? 8 : 4;
-  int waves = (dv + ML_COLS - 1) / ML_COLS;
-  if (waves > max_waves) waves = max_waves;
-  const size_t lds = ((size_t)ML_TB * (2 * rpl * ML_RG + dv) + 2 * ML_TB) * sizeof(float);
-  TI_REQUIRE(lds <= 64 * 1024, "mlstm: value size %d needs %zu bytes of LDS", dv, lds);
-  dim3 grid(n_entries, heads);
-#define ML_GO(R, T)                                                                                                   \
-  mlstm_scan_kernel<R, T><<<grid, waves * 64, lds, stream>>>(proj, ld, off_q, off_k, off_v, off_i, off_f, bias_i, bias_f, \
-                                                             state, slot_stride, entries, o, heads, dk, dv, cap, q_scale)
-  if (rpl == 8) ML_GO(8, 1024);
-  else if (rpl == 16) ML_GO(16, 1024);
-  else if (rpl == 32) ML_GO(32, 512);
-  else ML_GO(64, 256);
-#undef ML_GO
+  const int* chunks = nullptr;
+  float* chunk_buf = nullptr;
+  ML_LAUNCH(0, dim3(n_entries, heads));
+  TI_LAUNCH_CHECK();
+  return 0;
+}
+
+// The same with the entries' tokens cut into chunks that run side by side: chunks int32 [n_chunks][4] = (entry,
+// first row, tokens, 1 if the entry's first chunk + 2 if its last), in the entries' order; spans int32 [n_entries][2]
+// = (an entry's first chunk, its number of chunks); chunk_buf f32 [n_chunks][heads][dk dv + dk + 3] scratch.  Every
+// chunk alone, then the entries' chunks in order (element-wise), then every chunk from the state it starts from.
+// Where the chunks are cut changes the order of the sums: the same values up to rounding, not the same bits.
+extern "C" int ti_mlstm_scan_chunked(const float* proj, int ld, int off_q, int off_k, int off_v, int off_i, int off_f,
+                                     const float* bias_i, const float* bias_f, float* state, long slot_stride,
+                                     const int* entries, int n_entries, const int* chunks, int n_chunks, const int* spans,
+                                     float* chunk_buf, float* o, int heads, int dk, int dv, float cap, float q_scale,
+                                     hipStream_t stream) {
+  int rpl, waves;
+  size_t lds;
+  if (int rc = mlstm_shape(heads, dk, dv, cap, &rpl, &waves, &lds)) return rc;
+  TI_REQUIRE(chunks && spans && chunk_buf && n_chunks >= n_entries, "mlstm: %d chunks for %d entries, or no lists", n_chunks, n_entries);
+  if (n_entries == 0) return 0;
+  if (n_chunks > n_entries) {
+    ML_LAUNCH(1, dim3(n_chunks, heads));
+    const size_t elems = (size_t)dk * dv + dk;
+    const unsigned slices = (unsigned)((elems + 256 * 8 - 1) / (256 * 8));
+    mlstm_combine_kernel<<<dim3(n_entries, heads, slices), 256, 0, stream>>>(state, slot_stride, entries, spans, chunk_buf, heads,
+                                                                            dk, dv);
+  }
+  ML_LAUNCH(2, dim3(n_chunks, heads));
   TI_LAUNCH_CHECK();
   return 0;
 }

@@ -121,6 +121,13 @@ int ti_qkv_split_write(int dtype, const float* qkv, const int* pos, const int* s
 int ti_mlstm_scan(const float* proj, int ld, int off_q, int off_k, int off_v, int off_i, int off_f, const float* bias_i,
                   const float* bias_f, float* state, long slot_stride, const int* entries, int n_entries, float* o,
                   int heads, int dk, int dv, float cap, float q_scale, hipStream_t stream);
+// the same with long portions cut into chunks that run side by side: chunks int32 [n_chunks][4] = (entry, first row,
+// tokens, 1 if the entry's first chunk + 2 if its last) in the entries' order, spans int32 [n_entries][2] = (an entry's
+// first chunk, its chunks), chunk_buf f32 [n_chunks][heads][dk dv + dk + 3] scratch.  The same values up to rounding.
+int ti_mlstm_scan_chunked(const float* proj, int ld, int off_q, int off_k, int off_v, int off_i, int off_f,
+                          const float* bias_i, const float* bias_f, float* state, long slot_stride, const int* entries,
+                          int n_entries, const int* chunks, int n_chunks, const int* spans, float* chunk_buf, float* o,
+                          int heads, int dk, int dv, float cap, float q_scale, hipStream_t stream);
 // out = o / rms(o per head) * w * sigmoid(gate), gate in rows of ld floats from column off_g on
 int ti_gated_head_norm(int out_dtype, const float* o, const float* gate, int ld, int off_g, const float* w, void* out,
                        int M, int heads, int dv, float eps, hipStream_t stream);

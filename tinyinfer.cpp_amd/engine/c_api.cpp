@@ -1248,8 +1248,11 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
     c.v = (int)num(7);
     c.i = (int)num(8);
     c.f = (int)num(9);
+    // optional: chunks [n][4] and spans [R][2] (tensors 6 and 7): the chunked form
+    const bool chunked = n_t > 7 && arg(6).defined();
     ops.mlstm_scan(arg(0), c, arg(1), arg(2), arg(3), iptr(4), (int)arg(4).shape[0], arg(5), (int)num(0), (int)num(1), (int)num(2),
-                   (float)num(3), (float)num(4));
+                   (float)num(3), (float)num(4), chunked ? iptr(6) : nullptr, chunked ? (int)arg(6).shape[0] : 0,
+                   chunked ? iptr(7) : nullptr, chunked ? &workspace_of(&ops) : nullptr);
   } else if (op == "gated_head_norm") {
     // o, proj, w, out; gate column, eps, heads, dv
     ops.gated_head_norm(arg(0), arg(1), (int)num(0), arg(2), (float)num(1), arg(3), (int)num(2), (int)num(3));

@@ -334,8 +334,11 @@ class Ops {
   // The mLSTM cell over each entry's tokens, from and into its state slot.  proj f32 [M, ld] with the heads' q, k, v and
   // gate pre-activations from the given columns on; state f32 [slots][heads][dk dv + dk + 1]; o f32 [M, heads dv]
   struct MlstmColumns { int q = 0, k = 0, v = 0, i = 0, f = 0; };
+  // chunks (device int32 [n_chunks][4] = (entry, first row, tokens, 1: the entry's first chunk + 2: its last)) and spans
+  // ([n_entries][2] = (first chunk, chunks)): long portions run as chunks side by side, through scratch of `ws`
   void mlstm_scan(const Tensor& proj, const MlstmColumns& cols, const Tensor& bias_i, const Tensor& bias_f, const Tensor& state,
-                  const int* entry_meta, int n_entries, const Tensor& o, int heads, int dk, int dv, float cap, float q_scale);
+                  const int* entry_meta, int n_entries, const Tensor& o, int heads, int dk, int dv, float cap, float q_scale,
+                  const int* chunks = nullptr, int n_chunks = 0, const int* spans = nullptr, Workspace* ws = nullptr);
   // out = o / rms(o per head) * w * sigmoid(gate columns of proj), in the compute dtype
   void gated_head_norm(const Tensor& o, const Tensor& proj, int gate_col, const Tensor& w, float eps, const Tensor& out,
                        int heads, int dv);

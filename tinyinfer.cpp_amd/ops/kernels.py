@@ -343,9 +343,11 @@ class Ops:
         self._call("attention_capped", [q, pool, table, positions, slots, out],
                    [heads, kv_heads, dk, dv, scale, softcap, int(window or 0)])
 
-    def mlstm_scan(self, proj, bias_i, bias_f, state, entries, o, heads, dk, dv, cap, q_scale, columns):
-        """entries int32 [R, 4] = (first row, tokens, -, state slot); columns = (q, k, v, i, f) of proj."""
-        self._call("mlstm_scan", [proj, bias_i, bias_f, state, entries, o], [heads, dk, dv, cap, q_scale] + list(columns))
+    def mlstm_scan(self, proj, bias_i, bias_f, state, entries, o, heads, dk, dv, cap, q_scale, columns, chunks=None, spans=None):
+        """entries int32 [R, 4] = (first row, tokens, -, state slot); columns = (q, k, v, i, f) of proj.  chunks int32
+        [n, 4] = (entry, first row, tokens, 1: the entry's first chunk + 2: its last) and spans int32 [R, 2] = (first
+        chunk, chunks): the entries' tokens run as chunks side by side."""
+        self._call("mlstm_scan", [proj, bias_i, bias_f, state, entries, o, chunks, spans], [heads, dk, dv, cap, q_scale] + list(columns))
 
     def gated_head_norm(self, o, proj, gate_col, w, eps, out, heads, dv):
         self._call("gated_head_norm", [o, proj, w, out], [gate_col, eps, heads, dv])

@@ -941,8 +941,9 @@ void Ops::attention_capped(const Tensor& q, const Tensor& pool, const CacheView&
 }
 
 void Ops::mlstm_scan(const Tensor& proj, const MlstmColumns& cols, const Tensor& bias_i, const Tensor& bias_f, const Tensor& state,
-                     const int* entry_meta, int n_entries, const Tensor& o, int heads, int dk, int dv, float cap, float q_scale) {
-  TIMED("mlstm_scan " + dims(proj) + " entries=" + std::to_string(n_entries));
+                     const int* entry_meta, int n_entries, const Tensor& o, int heads, int dk, int dv, float cap, float q_scale,
+                     const int* chunks, int n_chunks, const int* spans, Workspace* ws) {
+  TIMED("mlstm_scan " + dims(proj) + " entries=" + std::to_string(n_entries) + (chunks ? " chunks=" + std::to_string(n_chunks) : ""));
   const int64_t per_head = (int64_t)dk * dv + dk + 1;
   require(proj.ndim == 2 && proj.dtype == DType::F32 && proj.contiguous(), "mlstm_scan: proj must be contiguous float32 [M, N]");
   const int64_t N = proj.shape[1];
@@ -957,6 +958,18 @@ void Ops::mlstm_scan(const Tensor& proj, const MlstmColumns& cols, const Tensor&
   require(o.dtype == DType::F32 && o.contiguous() && o.ndim == 2 && o.shape[0] == proj.shape[0] && o.shape[1] == (int64_t)heads * dv,
           "mlstm_scan: o " + o.describe() + " does not fit");
   require(entry_meta != nullptr || n_entries == 0, "mlstm_scan: no entry records");
+  if (chunks) {
+    require(spans && ws && n_chunks >= n_entries, "mlstm_scan: chunks need spans and a workspace");
+    float* scratch = (float*)ws->get("mlstm.chunk_buf", (size_t)n_chunks * heads * (size_t)(per_head + 2) * 4);
+    int rc = KERNEL("recurrent", ti_mlstm_scan_chunked)((const float*)proj.data, (int)N, cols.q, cols.k, cols.v, cols.i, cols.f,
+                                                        (const float*)bias_i.data, (const float*)bias_f.data, (float*)state.data,
+                                                        (long)(heads * per_head), entry_meta, n_entries, chunks, n_chunks, spans,
+                                                        scratch, (float*)o.data, heads, dk, dv, cap, q_scale,
+                                                        (hipStream_t)launch_stream());
+    check("recurrent", rc, "mlstm_scan(chunked)");
+    took("[chunked]");
+    return;
+  }
   int rc = KERNEL("recurrent", ti_mlstm_scan)((const float*)proj.data, (int)N, cols.q, cols.k, cols.v, cols.i, cols.f,
                                               (const float*)bias_i.data, (const float*)bias_f.data, (float*)state.data,
                                               (long)(heads * per_head), entry_meta, n_entries, (float*)o.data, heads, dk, dv, cap,

@@ -898,6 +898,36 @@ class MLSTM final : public MixerPart {
     n.state_shape = {heads, (int64_t)dk * dv + dk + 1};
     return n;
   }
+  // A step with a long portion: every entry's tokens in chunks of CHUNK (the cell's recurrence runs inside the chunks
+  // side by side and from chunk to chunk element-wise), from CHUNK_FROM tokens on, where three chunks or more make up
+  // for walking the tokens twice.  The lists are the same for every mLSTM of the model; the first one builds them.
+  static constexpr int CHUNK = 64, CHUNK_FROM = 192;
+  void plan(StepPlan& plan) const override {
+    if (plan.decode_only() || plan.has("mlstm.chunks")) return;
+    const auto& entries = plan.entries();
+    int longest = 0;
+    size_t n_chunks = 0;
+    for (const auto& e : entries) {
+      longest = std::max(longest, e.n_tokens);
+      n_chunks += (size_t)(e.n_tokens + CHUNK - 1) / CHUNK;
+    }
+    if (longest < CHUNK_FROM) return;
+    int* chunks = plan.ints("mlstm.chunks", 4 * n_chunks);
+    int* spans = plan.ints("mlstm.spans", 2 * entries.size());
+    int c = 0;
+    for (size_t i = 0; i < entries.size(); ++i) {
+      const auto& e = entries[i];
+      const int n = (e.n_tokens + CHUNK - 1) / CHUNK;
+      spans[2 * i] = c;
+      spans[2 * i + 1] = n;
+      for (int k = 0; k < n; ++k, ++c) {
+        chunks[4 * c] = (int)i;
+        chunks[4 * c + 1] = e.row0 + k * CHUNK;
+        chunks[4 * c + 2] = std::min(CHUNK, e.n_tokens - k * CHUNK);
+        chunks[4 * c + 3] = (k == 0 ? 1 : 0) | (k == n - 1 ? 2 : 0);
+      }
+    }
+  }
   void run(StepContext& ctx, const Rows& h, const Tensor& out, Ops::Epilogue epi) {
     const int64_t M = h.t.shape[0];
     Tensor proj = ctx.buf("mlstm.proj", DType::F32, {M, width});
@@ -912,7 +942,8 @@ class MLSTM final : public MixerPart {
     cols.i = (int)(2 * nq + 2 * nv);
     cols.f = cols.i + heads;
     ctx.ops.mlstm_scan(proj, cols, b_i, b_f, state, ctx.entry_meta, (int)ctx.entries.size(), o, heads, dk, dv, cap,
-                       (float)(1.0 / std::sqrt((double)dk)));
+                       (float)(1.0 / std::sqrt((double)dk)), ctx.planned("mlstm.chunks"), (int)(ctx.planned_size("mlstm.chunks") / 4),
+                       ctx.planned("mlstm.spans"), &ctx.ws);
     Tensor a = ctx.buf("mlstm.gated", ctx.act_dtype, {M, nv});
     ctx.ops.gated_head_norm(o, proj, (int)(2 * nq + nv), norm_w, eps, a, heads, dv);
     ctx.ops.linear(a, w_o, out, epi, epi == Ops::Add);
