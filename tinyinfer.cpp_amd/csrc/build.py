@@ -49,10 +49,37 @@ SOURCES: Dict[str, str] = _discover()
 ON_DEMAND = ("measure",)
 
 
-def libraries_for(dtype: str) -> List[str]:
+# libraries that only some architectures call into (by the name config.json gives the architecture); every other
+# library serves them all
+ONLY_FOR = {"pointwise": ("Miterax",), "recurrent": ("Miterax",)}
+
+
+def libraries_for(dtype: str, architecture: str = None) -> List[str]:
     """The kernel libraries a model of this dtype needs: every one except those whose name ends in `_bf16`
-    when the engine runs in float32 (what a first call compiles)."""
-    return [n for n in SOURCES if n not in ON_DEMAND and (dtype == "bfloat16" or not n.endswith("_bf16"))]
+    when the engine runs in float32 (what a first call compiles).  With the architecture's name, the libraries
+    that only other architectures use are left out as well."""
+    names = [n for n in SOURCES if n not in ON_DEMAND and (dtype == "bfloat16" or not n.endswith("_bf16"))]
+    if architecture is not None:
+        names = [n for n in names if n not in ONLY_FOR or architecture in ONLY_FOR[n]]
+    return names
+
+
+def architecture_of(model_dir: str):
+    """The architecture's name in a model folder's config.json (None if it cannot be read: the caller then builds
+    for every architecture)."""
+    import json
+    try:
+        with open(os.path.join(model_dir, "config.json")) as f:
+            d = json.load(f)
+    except (OSError, ValueError):
+        return None
+    for key in ("architectures", "model_type", "architecture"):
+        v = d.get(key) if isinstance(d, dict) else None
+        if isinstance(v, list) and v and isinstance(v[0], str):
+            return v[0]
+        if isinstance(v, str):
+            return v
+    return None
 
 
 # the host library (configuration, weights, parts, cache manager, step function, scheduler, sampler
