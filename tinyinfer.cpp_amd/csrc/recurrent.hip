@@ -45,8 +45,12 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, 
   float* lq = lds;                        // [ML_TB][DP]
   float* lk = lq + ML_TB * DP;            // [ML_TB][DP]
   float* lv = lk + ML_TB * DP;            // [ML_TB][dv]
-  float* lgi = lv + ML_TB * dv;           // [ML_TB]
-  float* lgf = lgi + ML_TB;               // [ML_TB]
+  float* lgi = lv + ML_TB * dv;           // [ML_TB] log input gates
+  float* lgf = lgi + ML_TB;               // [ML_TB] log forget gates
+  float* lm = lgf + ML_TB;                // [ML_TB] the running maximum after each token
+  float* ldc = lm + ML_TB;                // [ML_TB] exp(f + m before - m after): what the memory keeps
+  float* ltk = ldc + ML_TB;               // [ML_TB] exp(i - m after): what the token adds
+  float* lem = ltk + ML_TB;               // [ML_TB] exp(-m after)
   const int unit = blockIdx.x, h = blockIdx.y;
   int e = unit, row0, n_tok, flags = 3;
   if (MODE == 0) {
@@ -73,7 +77,12 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, 
   float* S_dst = (MODE == 0 || (MODE == 2 && last)) ? slot_base : (MODE == 1 ? cb : nullptr);
   const int ov = heads * dv;
   const int span = n_waves * ML_COLS;
-  float S[RPL], nn[RPL];
+  // n is a vector, not a matrix: the 16 lanes that share a quarter of the rows split that quarter's n between them
+  // (NPL rows a lane) and add their shares of n . q up over the whole wavefront
+  constexpr int NPL = RPL >= ML_COLS ? RPL / ML_COLS : 1;
+  const bool n_lane = c * NPL < RPL;                 // (a quarter of fewer than 16 rows leaves lanes without one)
+  const int n_row0 = rg * RPL + c * NPL;
+  float S[RPL], nn[NPL];
   float m = 0.f, F = 0.f;
   for (int j0 = 0; j0 < dv; j0 += span) {
     const int j = j0 + wave * ML_COLS + c;
@@ -82,8 +91,9 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, 
     for (int i = 0; i < RPL; ++i) {
       const int r = rg * RPL + i;
       S[i] = (MODE != 1 && active && r < dk) ? S_src[(size_t)r * dv + j] : 0.f;
-      nn[i] = (MODE != 1 && r < dk) ? S_src[(size_t)dk * dv + r] : 0.f;
     }
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) nn[i] = (MODE != 1 && n_lane && n_row0 + i < dk) ? S_src[(size_t)dk * dv + n_row0 + i] : 0.f;
     m = (MODE == 1) ? -INFINITY : *m_src;
     F = 0.f;
     for (int t0 = 0; t0 < n_tok; t0 += ML_TB) {
@@ -106,16 +116,31 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, 
         lgf[threadIdx.x] = log_sigmoid_f(cap * tanhf(af / cap));
       }
       __syncthreads();
+      // the maxima are a chain over the tokens (one thread walks it); the three exponentials of a token hang on
+      // nothing else, so a thread per token takes them off the loop that every lane walks
+      if (threadIdx.x == 0) {
+        float mm = m;
+        for (int t = 0; t < tb; ++t) {
+          mm = fmaxf(lgf[t] + mm, lgi[t]);
+          lm[t] = mm;
+        }
+      }
+      __syncthreads();
+      if ((int)threadIdx.x < tb) {
+        const int t = threadIdx.x;
+        const float before = t ? lm[t - 1] : m, after = lm[t];
+        ldc[t] = expf(lgf[t] + before - after);
+        ltk[t] = expf(lgi[t] - after);
+        lem[t] = expf(-after);
+      }
+      __syncthreads();
       for (int t = 0; t < tb; ++t) {
-        const float ig = lgi[t], fg = lgf[t];
-        const float m_new = fmaxf(fg + m, ig);
-        const float decay = expf(fg + m - m_new), take = expf(ig - m_new);
-        m = m_new;
-        F += fg;
+        const float decay = ldc[t], take = ltk[t];
+        F += lgf[t];
         const float tv = active ? take * lv[t * dv + j] : 0.f;
         const float4* q4 = reinterpret_cast<const float4*>(lq + t * DP + rg * RPL);
         const float4* k4 = reinterpret_cast<const float4*>(lk + t * DP + rg * RPL);
-        float acc = 0.f, nq = 0.f;
+        float a4[4] = {0.f, 0.f, 0.f, 0.f};     // four sums side by side: shorter chains
 #pragma unroll
         for (int i = 0; i < RPL; i += 4) {
           const float4 qq = q4[i / 4], kk = k4[i / 4];
@@ -123,22 +148,26 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, 
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
             S[i + u] = fmaf(ka[u], tv, decay * S[i + u]);
-            nn[i + u] = fmaf(take, ka[u], decay * nn[i + u]);
-            if (MODE != 1) {
-              acc = fmaf(S[i + u], qa[u], acc);
-              nq = fmaf(nn[i + u], qa[u], nq);
-            }
+            if (MODE != 1) a4[u] = fmaf(S[i + u], qa[u], a4[u]);
           }
         }
+        float nq = 0.f;
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) {
+          const float kr = n_lane ? lk[t * DP + n_row0 + i] : 0.f;      // (rows beyond dk hold zeros)
+          nn[i] = fmaf(take, kr, decay * nn[i]);
+          if (MODE != 1) nq = fmaf(nn[i], n_lane ? lq[t * DP + n_row0 + i] : 0.f, nq);
+        }
         if (MODE != 1) {
+          float acc = (a4[0] + a4[1]) + (a4[2] + a4[3]);
           acc += __shfl_xor(acc, 16, TI_WAVE);
           acc += __shfl_xor(acc, 32, TI_WAVE);
-          nq += __shfl_xor(nq, 16, TI_WAVE);
-          nq += __shfl_xor(nq, 32, TI_WAVE);
-          const float denom = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
+          nq = group_sum<TI_WAVE>(nq);
+          const float denom = fmaxf(fabsf(nq), lem[t]) + 1e-6f;
           if (rg == 0 && active) o[(size_t)(row0 + t0 + t) * ov + h * dv + j] = acc / denom;
         }
       }
+      m = lm[tb - 1];
     }
     if (active && S_dst) {
 #pragma unroll
@@ -148,15 +177,13 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, 
       }
     }
   }
-  // n and m: every lane holds the same; one lane per quarter of the rows writes, after all have read
+  // n and m: every wavefront holds the same; the first one writes, after all have read
   __syncthreads();
-  if (S_dst && wave == 0 && c == 0) {
+  if (S_dst && wave == 0) {
 #pragma unroll
-    for (int i = 0; i < RPL; ++i) {
-      const int r = rg * RPL + i;
-      if (r < dk) S_dst[(size_t)dk * dv + r] = nn[i];
-    }
-    if (rg == 0) {
+    for (int i = 0; i < NPL; ++i)
+      if (n_lane && n_row0 + i < dk) S_dst[(size_t)dk * dv + n_row0 + i] = nn[i];
+    if (lane == 0) {
       S_dst[per_head - 1] = m;
       if (MODE == 1) S_dst[per_head] = F;
     }
@@ -177,27 +204,34 @@ mlstm_combine_kernel(const float* __restrict__ state, long slot_stride, const in
   const size_t per_head = (size_t)dk * dv + dk + 1, elems = per_head - 1, stride = per_head + 2;
   const float* slot_base = state + (size_t)entries[4 * e + 3] * slot_stride + (size_t)h * per_head;
   float m = slot_base[per_head - 1];
-  constexpr int PER = 8;            // elements a thread carries through the chunks
-  const size_t base = ((size_t)blockIdx.z * blockDim.x + threadIdx.x) * PER;
-  float run[PER];
+  const size_t idx = (size_t)blockIdx.z * blockDim.x + threadIdx.x;      // this thread's element of (S, n)
+  const bool mine = idx < elems;
+  float run = mine ? slot_base[idx] : 0.f;
+  float* cb0 = chunk_buf + ((size_t)first * heads + h) * stride;
+  const size_t step = (size_t)heads * stride;                            // from a chunk to the next
+  // what the chunks added alone does not hang on the running state: four chunks' loads go out together
+  for (int c0 = 0; c0 < n; c0 += 4) {
+    float loc[4], m_c[4], F_c[4];
 #pragma unroll
-  for (int k = 0; k < PER; ++k) run[k] = base + k < elems ? slot_base[base + k] : 0.f;
-  for (int cidx = 0; cidx < n; ++cidx) {
-    float* cb = chunk_buf + ((size_t)(first + cidx) * heads + h) * stride;
-    const float m_c = cb[per_head - 1], F_c = cb[per_head];
-    float loc[PER];
+    for (int k = 0; k < 4; ++k) {
+      const int cidx = c0 + k < n ? c0 + k : n - 1;
+      const float* cb = cb0 + (size_t)cidx * step;
+      const bool adds = c0 + k + 1 < n;                                  // an entry's last chunk has left nothing
+      loc[k] = (mine && adds) ? cb[idx] : 0.f;
+      m_c[k] = adds ? cb[per_head - 1] : 0.f;
+      F_c[k] = adds ? cb[per_head] : 0.f;
+    }
 #pragma unroll
-    for (int k = 0; k < PER; ++k) loc[k] = (cidx + 1 < n && base + k < elems) ? cb[base + k] : 0.f;
-#pragma unroll
-    for (int k = 0; k < PER; ++k)
-      if (base + k < elems) cb[base + k] = run[k];
-    if (blockIdx.z == 0 && threadIdx.x == 0) cb[per_head + 1] = m;
-    if (cidx + 1 < n) {
-      const float m_new = fmaxf(F_c + m, m_c);
-      const float a = expf(F_c + m - m_new), b = expf(m_c - m_new);
-#pragma unroll
-      for (int k = 0; k < PER; ++k) run[k] = fmaf(b, loc[k], a * run[k]);
-      m = m_new;
+    for (int k = 0; k < 4; ++k) {
+      if (c0 + k >= n) break;
+      float* cb = cb0 + (size_t)(c0 + k) * step;
+      if (mine) cb[idx] = run;
+      if (idx == 0) cb[per_head + 1] = m;
+      if (c0 + k + 1 < n) {
+        const float m_new = fmaxf(F_c[k] + m, m_c[k]);
+        run = fmaf(expf(m_c[k] - m_new), loc[k], expf(F_c[k] + m - m_new) * run);
+        m = m_new;
+      }
     }
   }
 }
@@ -210,7 +244,7 @@ static int mlstm_shape(int heads, int dk, int dv, float cap, int* rpl, int* wave
   const int max_waves = *rpl <= 16 ? 16 : *rpl == 32 ? 8 : 4;
   *waves = (dv + ML_COLS - 1) / ML_COLS;
   if (*waves > max_waves) *waves = max_waves;
-  *lds = ((size_t)ML_TB * (2 * *rpl * ML_RG + dv) + 2 * ML_TB) * sizeof(float);
+  *lds = ((size_t)ML_TB * (2 * *rpl * ML_RG + dv) + 6 * ML_TB) * sizeof(float);
   TI_REQUIRE(*lds <= 64 * 1024, "mlstm: value size %d needs %zu bytes of LDS", dv, *lds);
   return 0;
 }
@@ -268,7 +302,7 @@ extern "C" int ti_mlstm_scan_chunked(const float* proj, int ld, int off_q, int o
   if (n_chunks > n_entries) {
     ML_LAUNCH(1, dim3(n_chunks, heads));
     const size_t elems = (size_t)dk * dv + dk;
-    const unsigned slices = (unsigned)((elems + 256 * 8 - 1) / (256 * 8));
+    const unsigned slices = (unsigned)((elems + 255) / 256);
     mlstm_combine_kernel<<<dim3(n_entries, heads, slices), 256, 0, stream>>>(state, slot_stride, entries, spans, chunk_buf, heads,
                                                                             dk, dv);
   }

@@ -843,7 +843,7 @@ class MLSTM final : public MixerPart {
     if (heads <= 0 || dk <= 0 || dv <= 0 || hidden <= 0) throw ConfigError("mlstm: sizes must be positive");
     if (dk > 256) throw ConfigError("mlstm: a key size of " + std::to_string(dk) + " is not served (up to 256)");
     const int padded = dk <= 32 ? 32 : dk <= 64 ? 64 : dk <= 128 ? 128 : 256;      // the rows the scan kernel holds
-    if (2 * padded + dv > 1020)
+    if (2 * padded + dv > 1016)
       throw ConfigError("mlstm: a value size of " + std::to_string(dv) + " beside a key size of " + std::to_string(dk) +
                         " is not served (the scan stages sixteen tokens' q, k and v in 64 KB)");
     if (!(cap > 0.f)) throw ConfigError("mlstm: gate_cap must be positive");
