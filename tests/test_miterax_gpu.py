@@ -523,6 +523,53 @@ def test_greedy_generation_through_the_entry_point(folders, use_graph):
         assert g[:n] == toks[len(p):], (p[:3], g, toks[len(p):])
 
 
+def plain_greedy(config, w, prompt, n_new):
+    """(generated ids, how many of them stand clear of a tie within rounding)."""
+    toks, sure = list(prompt), 0
+    for k in range(n_new):
+        logits = plain.forward(config, w, toks)[-1]
+        best = int(np.argmax(logits))
+        if sure == k and logits[best] - np.partition(logits, -2)[-2] > 1e-3:
+            sure = k + 1
+        toks.append(best)
+    return toks[len(prompt):], sure
+
+
+def test_command_line_generates_from_a_miterax_folder(folders):
+    """bin/tinyinfer picks the model by config.json: token ids in, the plain model's greedy tokens out; with --cuda-graph too."""
+    import os
+    import subprocess
+    import sys
+    folder, requests, _, w = folders("noloop")
+    config = mm.CONFIGS["noloop"]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p1, p2 = requests["b"][:11], requests["d"][:4]
+    for extra in ([], ["--cuda-graph"]):
+        run = subprocess.run([sys.executable, os.path.join(root, "bin", "tinyinfer"), "-m", folder, "-n", "6", "-p", ",".join(map(str, p1)),
+                              "-p", " ".join(map(str, p2)), "--dtype", "float32", "--max-seq", "64"] + extra,
+                             capture_output=True, text=True, timeout=300)
+        assert run.returncode == 0, run.stderr[-2000:]
+        outputs = [l[len("[output] "):].split() for l in run.stdout.split("\n") if l.startswith("[output] ")]
+        assert len(outputs) == 2
+        for p, got in zip((p1, p2), outputs):
+            want, sure = plain_greedy(config, w, p, 6)
+            assert [int(t) for t in got][:sure] == want[:sure], (got, want)
+
+
+def test_random_weights_drawn_on_the_device_run(tmp_path):
+    """A config.json alone: the parts' declared distributions give a model that steps (what the bench tool measures)."""
+    from tinyinfer_amd.engine import Engine, StepEntry
+    for name in ("loop3", "odd"):
+        engine = Engine.from_config(mm.CONFIGS[name], seed=3, dtype="bfloat16", page_size=16, max_tokens=256, max_requests=2, max_seq=256)
+        toks = random_tokens(70, mm.CONFIGS[name]["vocab"], 1)
+        a = engine.step([StepEntry("x", toks, [69])]).cpu().numpy()
+        engine.release("x")
+        b = np.concatenate([engine.step([StepEntry("y", toks[:69], [])]) is None and np.zeros((0, a.shape[1])),
+                            engine.step([StepEntry("y", toks[69:], [0])]).cpu().numpy()])
+        assert np.isfinite(a).all() and a.std() > 0
+        assert np.abs(a - b).max() < 0.05 * max(1e-6, np.abs(a).max())
+
+
 def test_trace_replay_program(folders, tmp_path):
     """The replay program on a Miterax folder: it picks the model by config.json and writes the logits the engine gives."""
     import os
