@@ -257,6 +257,115 @@ def case_head_bandwidth(ops, rng) -> int:
                 f"  {us:6.1f} us  {N * K * 2 / us / 1e3:6.0f} GB/s")
 
 
+def case_pointwise(ops, rng) -> int:
+    """The element-wise kernels of parallel layers: sinusoidal positions, xIELU, the scaled sum into the residual."""
+    fails = 0
+    H, pos = 48, np.array([0, 7, 640, 3000], dtype=np.int32)
+    inv = np.array([10000.0 ** (-2.0 * i / H) for i in range(H // 2)], dtype=np.float32)
+    x0 = rng.normal(size=(len(pos), H)).astype(np.float32)
+    x = _dev(x0)
+    ops.add_sinusoid(x, _dev(pos), _dev(inv))
+    angle = pos[:, None].astype(np.float64) * inv[None, :].astype(np.float64)
+    want = x0.astype(np.float64)
+    want[:, 0::2] += np.sin(angle)
+    want[:, 1::2] += np.cos(angle)
+    fails += _say("sinusoidal positions added (32-bit angles)", float(np.abs(_f64(x) - want).max()), 5e-4)
+    z = (rng.normal(size=(16, 64)) * 3).astype(np.float32)
+    u, v = 0.4, -0.6
+    sp = lambda t: math.log1p(math.exp(t))      # noqa: E731
+    zz = z.astype(np.float64)
+    want = np.where(zz > 0, sp(u) * zz * zz + 0.5 * zz, (0.5 + sp(v)) * (np.expm1(np.minimum(zz, 0)) - np.minimum(zz, 0)) + 0.5 * zz)
+    for dt, tol in ((torch.float32, 1e-4), (torch.bfloat16, 0.2)):
+        out = torch.empty(16, 64, device="cuda", dtype=dt)
+        ops.xielu(_dev(z), _dev(np.array([u, v], dtype=np.float32)), out)
+        fails += _say(f"xIELU 16x64 -> {str(dt).split('.')[-1]}", float(np.abs(_f64(out) - want).max()), tol)
+    a, b = rng.normal(size=(16, 48)).astype(np.float32), rng.normal(size=(16, 48)).astype(np.float32)
+    sa, sb = rng.normal(size=48).astype(np.float32), rng.normal(size=48).astype(np.float32)
+    x0 = rng.normal(size=(16, 48)).astype(np.float32)
+    x = _dev(x0)
+    ops.scaled_add(x, _dev(a), _dev(sa), _dev(b), _dev(sb))
+    want = x0.astype(np.float64) + a.astype(np.float64) * sa + b.astype(np.float64) * sb
+    fails += _say("scaled sum of two branches into the residual", float(np.abs(_f64(x) - want).max()), 1e-5)
+    return fails
+
+
+def case_capped_attention(ops, rng, nh, nkv, dk, dv, T, dtype) -> int:
+    """q/k/v split with a query temperature into pages (K [kv][P][dk] | V [kv][dv][P]), then soft-capped attention of every row."""
+    P, cap, coef, every, scale = 16, 5.0, 0.3, 4, 1.0 / math.sqrt(dk)
+    q, k, v = rng.normal(size=(T, nh, dk)) * 1.5, rng.normal(size=(T, nkv, dk)), rng.normal(size=(T, nkv, dv))
+    qkv = np.concatenate([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], axis=1).astype(np.float32)
+    pages = -(-T // P)
+    table = rng.permutation(pages + 2)[:pages].astype(np.int32)[None, :]
+    pool = torch.zeros(pages + 2, nkv, P, dk + dv, device="cuda", dtype=dtype)
+    q_out = torch.empty(T, nh * dk, device="cuda", dtype=dtype)
+    pos, slots = _dev(np.arange(T, dtype=np.int32)), _dev(np.zeros(T, dtype=np.int32))
+    ops.qkv_split_write(_dev(qkv), pos, slots, _dev(table), pool, q_out, nh, nkv, dk, dv, coef, every)
+    out = torch.empty(T, nh * dv, device="cuda", dtype=dtype)
+    ops.attention_capped(q_out, pool, _dev(table), pos, slots, out, nh, nkv, dk, dv, scale, cap)
+    rnd = _bf16 if dtype == torch.bfloat16 else (lambda t: np.asarray(t, dtype=np.float32).astype(np.float64))
+    temp = np.array([1 + coef * math.log((p + 1) // every + 1) for p in range(T)])
+    qt, kr, vr = _f64(q_out).reshape(T, nh, dk), rnd(k), rnd(v)
+    err_q = float(np.abs(qt - rnd(q * temp[:, None, None])).max() / np.abs(qt).max())
+    want = np.zeros((T, nh, dv))
+    for i in range(T):
+        for h in range(nh):
+            g = h // (nh // nkv)
+            s = cap * np.tanh((kr[: i + 1, g] @ qt[i, h]) * scale / cap)
+            p = np.exp(s - s.max())
+            want[i, h] = (p / p.sum()) @ vr[: i + 1, g]
+    name = f"capped attention {nh}/{nkv} heads, {dk}/{dv}, {T} tokens, {str(dtype).split('.')[-1]}"
+    fails = _say(name + ": q", err_q, 1e-5 if dtype == torch.float32 else 1e-2)
+    return fails + _say(name, float(np.abs(_f64(out).reshape(T, nh, dv) - want).max()), 1e-4 if dtype == torch.float32 else 2e-2)
+
+
+def case_mlstm(ops, rng, heads, dk, dv, lengths, chunk) -> int:
+    """The mLSTM scan over several requests (whole, and cut into chunks that run side by side), then the gated head norm."""
+    cap, N = 6.0, heads * (2 * dk + 2 * dv + 2)
+    cq, ck, cv, cg = 0, heads * dk, 2 * heads * dk, 2 * heads * dk + heads * dv
+    ci, cf = cg + heads * dv, cg + heads * dv + heads
+    M = sum(lengths)
+    proj = rng.normal(size=(M, N)).astype(np.float32)
+    bi, bf = rng.normal(size=heads).astype(np.float32), (rng.normal(size=heads) + 2).astype(np.float32)
+    entries, chunks, spans, row = [], [], [], 0
+    for e, n_tok in enumerate(lengths):
+        entries.append([row, n_tok, 0, e])
+        n = -(-n_tok // chunk)
+        spans.append([len(chunks), n])
+        chunks += [[e, row + j * chunk, min(chunk, n_tok - j * chunk), (j == 0) | 2 * (j == n - 1)] for j in range(n)]
+        row += n_tok
+    p = proj.astype(np.float64)
+    want = np.zeros((M, heads, dv))
+    for row0, n_tok, _, _ in entries:
+        for h in range(heads):
+            S, n, m = np.zeros((dk, dv)), np.zeros(dk), 0.0
+            for t in range(row0, row0 + n_tok):
+                q, k, v = p[t, cq + h * dk: cq + (h + 1) * dk] * float(np.float32(dk ** -0.5)), p[t, ck + h * dk: ck + (h + 1) * dk], p[t, cv + h * dv: cv + (h + 1) * dv]
+                ig = cap * math.tanh((p[t, ci + h] + bi[h]) / cap)
+                fz = cap * math.tanh((p[t, cf + h] + bf[h]) / cap)
+                fg = min(fz, 0.0) - math.log1p(math.exp(-abs(fz)))
+                m_new = max(fg + m, ig)
+                S = math.exp(fg + m - m_new) * S + math.exp(ig - m_new) * np.outer(k, v)
+                n = math.exp(fg + m - m_new) * n + math.exp(ig - m_new) * k
+                m = m_new
+                want[t, h] = (S.T @ q) / (max(abs(float(n @ q)), math.exp(-m)) + 1e-6)
+    fails = 0
+    o = None
+    for how in ("token by token", "in chunks"):
+        state = torch.zeros(len(lengths), heads, dk * dv + dk + 1, device="cuda")
+        o = torch.empty(M, heads * dv, device="cuda")
+        more = {} if how == "token by token" else dict(chunks=_dev(np.array(chunks, dtype=np.int32)), spans=_dev(np.array(spans, dtype=np.int32)))
+        ops.mlstm_scan(_dev(proj), _dev(bi), _dev(bf), state, _dev(np.array(entries, dtype=np.int32)), o, heads, dk, dv, cap, dk ** -0.5,
+                       (cq, ck, cv, ci, cf), **more)
+        err = float(np.abs(_f64(o).reshape(M, heads, dv) - want).max() / max(1.0, np.abs(want).max()))
+        fails += _say(f"mLSTM scan {heads} heads {dk}x{dv}, {lengths} tokens, {how}", err, 3e-4)
+    w = rng.normal(size=heads * dv).astype(np.float32)
+    out = torch.empty(M, heads * dv, device="cuda")
+    ops.gated_head_norm(o, _dev(proj), cg, _dev(w), 1e-5, out, heads, dv)
+    oo = _f64(o).reshape(M, heads, dv)
+    normed = (oo / np.sqrt((oo * oo).mean(-1, keepdims=True) + 1e-5)).reshape(M, -1) * w / (1 + np.exp(-p[:, cg: cg + heads * dv]))
+    return fails + _say("gated head norm", float(np.abs(_f64(out) - normed).max()), 1e-4)
+
+
 def run_selftest() -> int:
     if not torch.cuda.is_available():
         print("[selftest] no GPU: the kernels of this framework run on an AMD GPU (gfx950) only", flush=True)
@@ -275,6 +384,11 @@ def run_selftest() -> int:
     fails += case_attention(ops, rng, nh=16, nkv=8, hd=128, T=2, dtype=torch.float32)
     fails += case_attention(ops, rng, nh=16, nkv=8, hd=128, T=300, dtype=torch.bfloat16)
     fails += case_attention(ops, rng, nh=3, nkv=1, hd=48, T=40, dtype=torch.bfloat16)
+    fails += case_pointwise(ops, rng)
+    fails += case_capped_attention(ops, rng, nh=4, nkv=2, dk=24, dv=40, T=70, dtype=torch.float32)
+    fails += case_capped_attention(ops, rng, nh=6, nkv=1, dk=64, dv=16, T=130, dtype=torch.bfloat16)
+    fails += case_mlstm(ops, rng, heads=2, dk=32, dv=48, lengths=[150, 1, 70], chunk=64)
+    fails += case_mlstm(ops, rng, heads=1, dk=128, dv=128, lengths=[200], chunk=64)
     fails += case_embed_argmax_sample(ops, rng)
     fails += case_model_shapes(ops, rng)
     fails += case_head_bandwidth(ops, rng)
