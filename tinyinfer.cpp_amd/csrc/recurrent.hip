@@ -9,9 +9,11 @@
 // The gates come from pre-activations a (with a bias b): i = cap tanh((a_i + b_i) / cap),
 // f = logsigmoid(cap tanh((a_f + b_f) / cap)).  State, gates and everything else here is 32-bit.
 //
-// One workgroup per (request of the step, head).  A wavefront owns 16 columns of S; the four lanes
-// that share a column hold a quarter of its rows each, in registers, for all tokens of the step.  The
-// tokens' q, k, v and gates pass through LDS sixteen at a time.  Every element of S, n and o is
+// One workgroup per (request of the step, head).  A wavefront owns 64 / RG columns of S; the RG lanes
+// that share a column hold a share of its rows each (RPL of them), in registers, for all tokens of the
+// step.  The tokens' q, k, v and gates pass through LDS sixteen at a time.  Key sizes up to 64 take
+// RG = 4; larger ones RG = 8: half the rows a lane, twice the wavefronts, which hide a token's chain
+// of dependent operations better (a workgroup's wavefronts are all a compute unit runs).  Every element of S, n and o is
 // computed by the same sequence of operations whether its token came alone or in a portion, so a
 // sequence cut differently gives the same bits.
 #include "common.h"
@@ -19,8 +21,6 @@
 
 TI_ERROR_API
 
-#define ML_COLS 16   // columns of the memory per wavefront
-#define ML_RG 4      // lanes sharing a column
 #define ML_TB 16     // tokens staged at a time
 
 __device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
@@ -34,13 +34,14 @@ __device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) -
 // MODE 2: every chunk from that state (an entry of a single chunk: from its slot) with output; an entry's last chunk
 //         writes the slot.
 // chunk_buf per (chunk, head): S [dk][dv], n [dk], m of the chunk alone, F, m the chunk starts from.
-template <int RPL, int MAXT, int MODE>
+template <int RPL, int RG, int MAXT, int MODE>
 __global__ void __launch_bounds__(MAXT)
 mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, int off_v, int off_i, int off_f,
                   const float* __restrict__ bias_i, const float* __restrict__ bias_f, float* __restrict__ state,
                   long slot_stride, const int* __restrict__ entries, const int* __restrict__ chunks,
                   float* __restrict__ chunk_buf, float* __restrict__ o, int heads, int dk, int dv, float cap, float q_scale) {
-  constexpr int DP = RPL * ML_RG;   // rows, padded
+  constexpr int ML_COLS = TI_WAVE / RG;   // columns of the memory per wavefront
+  constexpr int DP = RPL * RG;            // rows, padded
   extern __shared__ __align__(16) float lds[];
   float* lq = lds;                        // [ML_TB][DP]
   float* lk = lq + ML_TB * DP;            // [ML_TB][DP]
@@ -65,7 +66,7 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, 
   const bool whole = (flags & 3) == 3, last = (flags & 2) != 0;
   if (MODE == 1 && last) return;          // nobody reads what an entry's last chunk adds alone
   const int slot = entries[4 * e + 3];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, rg = lane >> 4, c = lane & 15;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, rg = lane / ML_COLS, c = lane % ML_COLS;
   const int n_waves = blockDim.x >> 6;
   const size_t per_head = (size_t)dk * dv + dk + 1;
   float* slot_base = state + (size_t)slot * slot_stride + (size_t)h * per_head;
@@ -77,7 +78,7 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, 
   float* S_dst = (MODE == 0 || (MODE == 2 && last)) ? slot_base : (MODE == 1 ? cb : nullptr);
   const int ov = heads * dv;
   const int span = n_waves * ML_COLS;
-  // n is a vector, not a matrix: the 16 lanes that share a quarter of the rows split that quarter's n between them
+  // n is a vector, not a matrix: the lanes that share a share of the rows split that share's n between them
   // (NPL rows a lane) and add their shares of n . q up over the whole wavefront
   constexpr int NPL = RPL >= ML_COLS ? RPL / ML_COLS : 1;
   const bool n_lane = c * NPL < RPL;                 // (a quarter of fewer than 16 rows leaves lanes without one)
@@ -160,8 +161,8 @@ mlstm_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off_k, 
         }
         if (MODE != 1) {
           float acc = (a4[0] + a4[1]) + (a4[2] + a4[3]);
-          acc += __shfl_xor(acc, 16, TI_WAVE);
-          acc += __shfl_xor(acc, 32, TI_WAVE);
+#pragma unroll
+          for (int off = ML_COLS; off < TI_WAVE; off <<= 1) acc += __shfl_xor(acc, off, TI_WAVE);
           nq = group_sum<TI_WAVE>(nq);
           const float denom = fmaxf(fabsf(nq), lem[t]) + 1e-6f;
           if (rg == 0 && active) o[(size_t)(row0 + t0 + t) * ov + h * dv + j] = acc / denom;
@@ -240,29 +241,25 @@ static int mlstm_shape(int heads, int dk, int dv, float cap, int* rpl, int* wave
   TI_REQUIRE(heads > 0 && heads <= 65535 && dk >= 1 && dk <= 256 && dv >= 1, "mlstm: heads %d, key size %d (up to 256), value size %d",
              heads, dk, dv);
   TI_REQUIRE(cap > 0.f, "mlstm: the gates' cap must be positive");
-  *rpl = dk <= 32 ? 8 : dk <= 64 ? 16 : dk <= 128 ? 32 : 64;
-  const int max_waves = *rpl <= 16 ? 16 : *rpl == 32 ? 8 : 4;
-  *waves = (dv + ML_COLS - 1) / ML_COLS;
+  // rows a lane and lanes a column: 8 x 4, 16 x 4, 16 x 8, 32 x 8 for key sizes up to 32, 64, 128, 256
+  *rpl = dk <= 32 ? 8 : dk <= 128 ? 16 : 32;
+  const int rg = dk <= 64 ? 4 : 8, cols = 64 / rg;
+  const int max_waves = *rpl <= 16 ? 16 : 8;
+  *waves = (dv + cols - 1) / cols;
   if (*waves > max_waves) *waves = max_waves;
-  *lds = ((size_t)ML_TB * (2 * *rpl * ML_RG + dv) + 6 * ML_TB) * sizeof(float);
+  *lds = ((size_t)ML_TB * (2 * *rpl * rg + dv) + 6 * ML_TB) * sizeof(float);
   TI_REQUIRE(*lds <= 64 * 1024, "mlstm: value size %d needs %zu bytes of LDS", dv, *lds);
   return 0;
 }
 
-#define ML_LAUNCH(MODE, GRID)                                                                                          \
-  do {                                                                                                                 \
-    if (rpl == 8)                                                                                                      \
-      mlstm_scan_kernel<8, 1024, MODE><<<GRID, waves * 64, lds, stream>>>(proj, ld, off_q, off_k, off_v, off_i, off_f, bias_i, \
-          bias_f, state, slot_stride, entries, chunks, chunk_buf, o, heads, dk, dv, cap, q_scale);                     \
-    else if (rpl == 16)                                                                                                \
-      mlstm_scan_kernel<16, 1024, MODE><<<GRID, waves * 64, lds, stream>>>(proj, ld, off_q, off_k, off_v, off_i, off_f, bias_i, \
-          bias_f, state, slot_stride, entries, chunks, chunk_buf, o, heads, dk, dv, cap, q_scale);                     \
-    else if (rpl == 32)                                                                                                \
-      mlstm_scan_kernel<32, 512, MODE><<<GRID, waves * 64, lds, stream>>>(proj, ld, off_q, off_k, off_v, off_i, off_f, bias_i, \
-          bias_f, state, slot_stride, entries, chunks, chunk_buf, o, heads, dk, dv, cap, q_scale);                     \
-    else                                                                                                               \
-      mlstm_scan_kernel<64, 256, MODE><<<GRID, waves * 64, lds, stream>>>(proj, ld, off_q, off_k, off_v, off_i, off_f, bias_i, \
-          bias_f, state, slot_stride, entries, chunks, chunk_buf, o, heads, dk, dv, cap, q_scale);                     \
+#define ML_ARGS proj, ld, off_q, off_k, off_v, off_i, off_f, bias_i, bias_f, state, slot_stride, entries, chunks, chunk_buf, o, heads, dk, \
+                dv, cap, q_scale
+#define ML_LAUNCH(MODE, GRID)                                                                                  \
+  do {                                                                                                         \
+    if (dk <= 32) mlstm_scan_kernel<8, 4, 1024, MODE><<<GRID, waves * 64, lds, stream>>>(ML_ARGS);             \
+    else if (dk <= 64) mlstm_scan_kernel<16, 4, 1024, MODE><<<GRID, waves * 64, lds, stream>>>(ML_ARGS);       \
+    else if (dk <= 128) mlstm_scan_kernel<16, 8, 1024, MODE><<<GRID, waves * 64, lds, stream>>>(ML_ARGS);      \
+    else mlstm_scan_kernel<32, 8, 512, MODE><<<GRID, waves * 64, lds, stream>>>(ML_ARGS);                      \
   } while (0)
 
 // proj f32 [M, ld]: the projections of the step's rows; off_*: the columns where the heads' q [heads][dk],
