@@ -50,6 +50,12 @@ CONFIGS = {
                         mlstm(1, 130, 70, 20.0),
                         attention(2, 1, 7, 9, 0.4, softcap=50.0, coef=0.05, every=100, ff=8)],
                 loop=dict(start=1, stop=4, times=2)),
+    # a width that is no multiple of four (no 16-byte rows anywhere), tiny heads, an odd feed-forward, a loop over one layer
+    "width50": dict(architecture="Miterax", width=50, vocab=71, norm=dict(eps=1e-5),
+                    layers=[attention(2, 1, 10, 6, 0.31, softcap=7.0, coef=0.2, every=2, ff=30),
+                            mlstm(1, 5, 3, 4.0, ff=17),
+                            attention(4, 2, 3, 11, 0.5, softcap=1.5, coef=0.7, every=9)],
+                    loop=dict(start=1, stop=2, times=2)),
 }
 
 

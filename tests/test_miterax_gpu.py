@@ -415,7 +415,7 @@ def make_trace(mode, requests):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,page_size", [("loop3", 16), ("noloop", 4), ("wide", 16), ("odd", 32)])
+@pytest.mark.parametrize("name,page_size", [("loop3", 16), ("noloop", 4), ("wide", 16), ("odd", 32), ("width50", 8)])
 @pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
 def test_engine_matches_plain(folders, name, page_size, dtype, mode):
     folder, requests, want, _ = folders(name)
