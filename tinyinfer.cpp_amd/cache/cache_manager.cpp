@@ -19,7 +19,7 @@
 namespace tinyinfer {
 
 bool CacheNeed::operator==(const CacheNeed& o) const {
-  return kind == o.kind && kv_heads == o.kv_heads && head_dim == o.head_dim && value_dim() == o.value_dim() && window == o.window &&
+  return kind == o.kind && kv_heads == o.kv_heads && head_dim == o.head_dim && value_dim() == o.value_dim() && window == o.window && block == o.block &&
          state_shape == o.state_shape && row_shape == o.row_shape && rows_f32 == o.rows_f32;
 }
 
@@ -207,8 +207,11 @@ void CacheManager::reserve(int64_t req, int n_tokens) {
 }
 
 int CacheManager::first_needed_page(const Group& g, int next_pos) const {
-  if (g.need.window <= 0) return 0;
-  return std::max(0, next_pos - g.need.window + 1) / page_size;
+  // the first position that the token at next_pos (and every later one) still reads
+  int first = 0;
+  if (g.need.window > 0) first = std::max(first, next_pos - g.need.window + 1);
+  if (g.need.block > 0) first = std::max(first, next_pos / g.need.block * g.need.block);
+  return first / page_size;
 }
 
 void CacheManager::give_back_page(Group& g, int64_t req, int index) {
@@ -288,6 +291,12 @@ void CacheManager::commit_one_each(const std::vector<int64_t>& reqs) {
     r.length += 1;
     for (int gi : paged_) {
       Group& g = groups_[gi];
+      if (g.need.block > 0 && r.length % g.need.block == 0) {
+        // the next token opens a block: every page wholly before it goes back
+        auto& t = g.tables[q];
+        for (int i = 0; i < std::min(first_needed_page(g, r.length), (int)t.size()); ++i)
+          if (t[i] >= 0) give_back_page(g, q, i);
+      }
       if (g.need.window <= 0) continue;
       // a page falls behind the window only when the window's first position enters a new page
       const int lo = r.length - g.need.window + 1;

@@ -51,7 +51,10 @@ ON_DEMAND = ("measure",)
 
 # libraries that only some architectures call into (by the name config.json gives the architecture); every other
 # library serves them all
-ONLY_FOR = {"pointwise": ("Miterax",), "recurrent": ("Miterax",)}
+ONLY_FOR = {"pointwise": ("Miterax",), "recurrent": ("Miterax",), "residual": ("Mumasun",), "diff_attention": ("Mumasun",),
+            "moe": ("Mumasun",)}
+# ... and libraries that a named architecture never calls into
+NOT_FOR = {"attention_generic": ("Mumasun",), "attention_bf16": ("Mumasun",)}
 
 
 def libraries_for(dtype: str, architecture: str = None) -> List[str]:
@@ -60,7 +63,7 @@ def libraries_for(dtype: str, architecture: str = None) -> List[str]:
     that only other architectures use are left out as well."""
     names = [n for n in SOURCES if n not in ON_DEMAND and (dtype == "bfloat16" or not n.endswith("_bf16"))]
     if architecture is not None:
-        names = [n for n in names if n not in ONLY_FOR or architecture in ONLY_FOR[n]]
+        names = [n for n in names if (n not in ONLY_FOR or architecture in ONLY_FOR[n]) and architecture not in NOT_FOR.get(n, ())]
     return names
 
 
@@ -85,7 +88,7 @@ def architecture_of(model_dir: str):
 # the host library (configuration, weights, parts, cache manager, step function, scheduler, sampler
 # and the C interface the Python package binds): C++17, no device code
 PKG = os.path.dirname(HERE)
-HOST_SOURCES = ["config/json.cpp", "config/config.cpp", "config/miterax.cpp", "ops/ops.cpp", "parts/parts.cpp", "weights/weights.cpp",
+HOST_SOURCES = ["config/json.cpp", "config/config.cpp", "config/miterax.cpp", "config/mumasun.cpp", "ops/ops.cpp", "parts/parts.cpp", "weights/weights.cpp",
                 "models/model.cpp", "cache/cache_manager.cpp", "engine/engine.cpp", "engine/scheduler.cpp",
                 "sampling/sampler.cpp", "engine/c_api.cpp"]
 HOST_HEADERS = ["include/inference.h", "weights/weights.h", "csrc/tinyinfer_kernels.h"]

@@ -132,6 +132,46 @@ int ti_mlstm_scan_chunked(const float* proj, int ld, int off_q, int off_k, int o
 int ti_gated_head_norm(int out_dtype, const float* o, const float* gate, int ld, int off_g, const float* w, void* out,
                        int M, int heads, int dv, float eps, hipStream_t stream);
 
+// ---- libti_residual: layers that norm what a sublayer returns
+// x[m] (+)= y'[m] / sqrt(mean(y'[m]^2) + eps) * g; y'[m] = y[m], or with `gather` (int32 [M][n_gather]) the sum of
+// the rows y[gather[m][k]] in ascending k.  accumulate 0: x is overwritten (y may be x itself)
+int ti_norm_residual(float* x, const float* y, const float* g, const int* gather, int n_gather, int M, int H, float eps,
+                     int accumulate, hipStream_t stream);
+// out = x rounded to out_dtype
+int ti_round_rows(int out_dtype, const float* x, void* out, long n, hipStream_t stream);
+// x *= s
+int ti_scale(float* x, float s, long n, hipStream_t stream);
+
+// ---- libti_diff_attention: a short convolution over time with carried state, and differential attention
+// out[m, c] = sum_j taps[c][j] u(pos[m] - (K - 1) + j)[c]; u f32 [M, C] holds the step's rows, state f32
+// [slots][K - 1][C] the K - 1 rows before each entry's start (entries int32 [n][4] = (row0, tokens, start, slot);
+// entry_of[m]: the entry of row m), which the call then replaces by the last K - 1 rows up to the step's end
+int ti_short_conv(const float* u, const float* taps, float* state, const int* entries, int n_entries, const int* entry_of,
+                  const int* pos, float* out, int M, int C, int K, hipStream_t stream);
+// qkv f32 [M, n_head 2 dk + n_kv 2 dk + n_kv dv] (each query head and kv head holds two maps of dk): per map RMS
+// norm with the weights q_w / k_w [dk] (may be null), rotation of the first rot_dims entries (entry i with entry
+// i + rot_dims / 2; cos and sin times mag; rope_table [table_len][rot_dims / 2][2] may be null), q to q_out, k and v
+// into pages K [n_kv][P][2 dk] | V [n_kv][dv][P]
+int ti_diff_qk_prep(int dtype, const float* qkv, const float* q_w, const float* k_w, float eps, const float* inv_freq,
+                    const float* rope_table, int table_len, float mag, int rot_dims, const int* pos, const int* slot,
+                    const int* table, int table_stride, void* pool, void* q_out, int M, int n_head, int n_kv, int dk, int dv,
+                    int page_size, hipStream_t stream);
+// out[m, h] = (a1 - lambda a2) / rms(a1 - lambda a2) * out_scale, a1 and a2 the softmax attention of the head's two
+// maps over the keys that are not later than pos[m], in its block of `block` positions (0: none) and inside the window
+int ti_diff_attention_rows(int dtype, const void* q, const void* pool, const int* table, int table_stride, const int* pos,
+                           const int* slot, void* out, int M, int n_head, int n_kv, int dk, int dv, int page_size, float scale,
+                           int block, int window, float lambda, float eps, float out_scale, hipStream_t stream);
+
+// ---- libti_moe: a mixture of experts
+// scores (score_kind 0: sigmoid, 1: softmax over the experts) of h [M, W] against router f32 [E, W] in 32-bit; the `top`
+// largest per token (ties: the lower index) to ids int32 [M, top] and wts f32 [M, top] (renormalize: divided by their sum)
+int ti_moe_route(int dtype, const void* h, const float* router, int* ids, float* wts, int M, int W, int E, int top,
+                 int score_kind, int renormalize, hipStream_t stream);
+// y f32 [M, W] = sum_k down[e_k] relu(up[e_k] (s_k h))^2 (scale_input) or sum_k s_k down[e_k] relu(up[e_k] h)^2;
+// up [E][F][W], down [E][W][F] in the dtype of h
+int ti_moe_experts_rows(int dtype, const void* h, const int* ids, const float* wts, const void* up, const void* down, float* y,
+                        int M, int W, int F, int top, int scale_input, hipStream_t stream);
+
 // ---- libti_attention_bf16: the same on the matrix cores (head sizes 32, 64, 128; pages of 16 n rows)
 // rows of single tokens; n_splits > 1 needs part_o f32 [n_rows, n_head, n_splits, hd] and part_ml f32
 // [n_rows, n_head, n_splits, 2]

@@ -86,6 +86,7 @@ Json cache_need_json(const CacheNeed& n) {
     j.set("head_dim", n.head_dim);
     if (n.value_dim() != n.head_dim) j.set("v_dim", n.v_dim);
     j.set("window", n.window > 0 ? Json(n.window) : Json());
+    if (n.block > 0) j.set("block", n.block);
   } else if (n.kind == CacheNeed::PagedRows) {
     j.set("kind", "paged_rows");
     Json s = Json::array();
@@ -117,6 +118,7 @@ CacheNeed cache_need_from(const Json& c) {
     n.head_dim = (int)c.at("head_dim").as_int();
     n.v_dim = c.has("v_dim") ? (int)c.at("v_dim").as_int() : 0;
     n.window = c.has("window") ? (int)c.at("window").as_int() : 0;
+    n.block = c.has("block") ? (int)c.at("block").as_int() : 0;
   }
   return n;
 }

@@ -163,6 +163,9 @@ void register_architecture(const std::vector<std::string>& names, SpecBuilder bu
 // the Miterax decoder (config/miterax.cpp): its config.json read and validated, and its model as data
 Json miterax_typed_config(const Json& config);
 ModelSpec miterax_spec(const Json& config);
+// the Mumasun decoder (config/mumasun.cpp)
+Json mumasun_typed_config(const Json& config);
+ModelSpec mumasun_spec(const Json& config);
 // {"architecture": the registered name that matched, "config": the typed configuration (the input itself if
 // the architecture registered no reader)}; ConfigError as spec_from_config
 Json typed_config(const Json& config);
@@ -244,6 +247,8 @@ struct CacheNeed {
   // (a mixer with another kind of memory than keys and values).  State: a fixed size per request.
   enum Kind { PagedKV, State, PagedRows } kind = PagedKV;
   int kv_heads = 0, head_dim = 0, window = 0;    // PagedKV; window (PagedRows too) 0: every token is kept
+  int block = 0;                                 // paged: a token is read only from positions of its own block of this many
+                                                 // positions counted from 0 (0: no blocks); pages before the block go back
   int v_dim = 0;                                 // PagedKV: the size of a value where it is not head_dim (0: it is).  A page
                                                  // is then K [kv heads][P][head_dim] | V [kv heads][v_dim][P]
   int value_dim() const { return v_dim > 0 ? v_dim : head_dim; }
@@ -289,7 +294,8 @@ class Ops {
   void rmsnorm(const Tensor& x, const Tensor& w, float eps, const Tensor& out, const int* rows = nullptr, int64_t n_rows = 0);
   void rope_neox(const Tensor& x, const int* positions, const Tensor& inv_freq);      // in place on f32 [M, heads, hd]
   void rope_table(const Tensor& inv_freq, const Tensor& table);                       // f32 [n_pos, hd/2, 2]
-  struct Rotation { const float* inv_freq = nullptr; const float* table = nullptr; int table_len = 0; };
+  // dims: how many leading entries of a head are turned (0: all of them); mag: a factor on cosine and sine (the table holds it already)
+  struct Rotation { const float* inv_freq = nullptr; const float* table = nullptr; int table_len = 0; int dims = 0; float mag = 1.f; };
   struct CacheView { const int* table = nullptr; int table_width = 0; int page_size = 0; };
   void qk_norm_rope_kv_write(const Tensor& qkv, const float* q_w, const float* k_w, float eps, const Rotation& rot,
                              const int* positions, const int* slots, const CacheView& view, const Tensor& pool,
@@ -342,6 +348,35 @@ class Ops {
   // out = o / rms(o per head) * w * sigmoid(gate columns of proj), in the compute dtype
   void gated_head_norm(const Tensor& o, const Tensor& proj, int gate_col, const Tensor& w, float eps, const Tensor& out,
                        int heads, int dv);
+  // ---- layers that norm what a sublayer returns; short convolutions; differential attention; mixtures of experts
+  // x (+)= y / rms(y) * gain (32-bit; gain is the factor itself).  accumulate false: x is overwritten (y may be x).
+  // gather (device int32 [M][n_gather]): row m of y is the sum of the rows y[gather[m][k]], k ascending
+  void norm_residual(const Tensor& x, const Tensor& y, const Tensor& gain, float eps, bool accumulate, const int* gather = nullptr,
+                     int n_gather = 0);
+  void round_rows(const Tensor& x, const Tensor& out);                               // out = x in out's dtype
+  void scale(const Tensor& x, float s);                                              // x *= s (float32)
+  // out[m, c] = sum_j taps[c, j] u(position of m - (K - 1) + j)[c] over each entry's rows, the K - 1 rows before an
+  // entry's start taken from its state slot f32 [slots][K - 1][C]; the slot then gets the entry's last K - 1 rows
+  void short_conv(const Tensor& u, const Tensor& taps, const Tensor& state, const int* entry_meta, int n_entries,
+                  const int* entry_of, const int* positions, const Tensor& out);
+  // qkv f32 [M, heads 2 dk + kv_heads 2 dk + kv_heads dv] (two maps a head): per-map norm, rotation of the first
+  // rot.dims entries, q to q_out, k and v into pages K [kv][P][2 dk] | V [kv][dv][P]
+  void diff_qk_prep(const Tensor& qkv, const float* q_w, const float* k_w, float eps, const Rotation& rot, const int* positions,
+                    const int* slots, const CacheView& view, const Tensor& pool, const Tensor& q_out, int heads, int kv_heads,
+                    int dk, int dv);
+  // differential attention of every row over such pages: (a1 - lambda a2) / rms * out_scale per head; a key is visible
+  // inside the query's block of `block` positions (0: no blocks) and window (0: none)
+  void diff_attention(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
+                      const Tensor& out, int heads, int kv_heads, int dk, int dv, float scale, int block, int window, float lambda,
+                      float eps, float out_scale);
+  enum RouterScore { Sigmoid = 0, Softmax = 1 };
+  // the `top` experts with the largest scores of h against router f32 [E, W]: ids int32 [M, top], wts f32 [M, top]
+  void moe_route(const Tensor& h, const Tensor& router, const Tensor& ids, const Tensor& wts, int top, RouterScore score,
+                 bool renormalize);
+  // y f32 [M, W] = sum over a token's experts of down_e relu(up_e h)^2, the weight on the expert's input or output;
+  // up [E F, W], down [E W, F]
+  void moe_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, const Tensor& up, const Tensor& down, const Tensor& y,
+                   int experts, bool scale_input);
   void argmax(const Tensor& logits, int* out);
   void sample(const Tensor& logits, const float* temperature, const int* top_k, const float* top_p, const float* uniform,
               int* out);
@@ -522,6 +557,7 @@ class StepContext {
 //   norm       forward(ctx, x, rows, n_rows, lazy)   -> Rows in the compute dtype
 //   pos        fused(rot) / apply(ctx, q, k)         rotation in the fused kernels, or in place on f32 views
 //   mixer      forward(ctx, h, x)                    adds its output into x
+//   filter     forward(ctx, u, out)                  out f32 [M, C] from u f32 [M, C] over each entry's rows in time
 //   ffn        forward(ctx, h, x)                    adds its output into x
 //   block      forward(ctx, x)                       arranges its parts around x
 //   head       forward(ctx, h) -> logits f32 [N, V]
@@ -558,7 +594,12 @@ class EmbeddingPart : public Part { public: using Part::Part; const char* family
   virtual void forward(StepContext& ctx, const Tensor& x) = 0; };
 class NormPart : public Part { public: using Part::Part; const char* family() const override { return "norm"; }
   virtual Rows forward(StepContext& ctx, const Tensor& x, const int* rows = nullptr, int64_t n_rows = 0, bool lazy = false) = 0;
-  virtual bool can_be_lazy() const { return false; } };
+  virtual bool can_be_lazy() const { return false; }
+  // x (+)= norm(y), both f32 [M, dim], in 32-bit: for arrangements that norm what a sublayer returns (y may be x itself
+  // when nothing is accumulated)
+  virtual bool can_add() const { return false; }
+  virtual void forward_add(StepContext& ctx, const Tensor& y, const Tensor& x, bool accumulate, const int* gather = nullptr,
+                           int n_gather = 0); };
 class PositionPart : public Part { public: using Part::Part; const char* family() const override { return "pos"; }
   virtual bool fused(Ops::Rotation& rot) const { return false; }    // arguments for the fused q/k kernels
   virtual bool additive() const { return false; }                   // an encoding added to the residual behind the embedding ...
@@ -570,6 +611,9 @@ class MixerPart : public Part { public: using Part::Part; const char* family() c
   virtual bool can_store() const { return false; }
   virtual void forward_store(StepContext& ctx, const Rows& h, const Tensor& y);
   virtual bool takes_lazy_norm() const { return false; } };        // h goes into exactly one Ops::linear
+// an operation along time on every channel of the step's rows, with what it must remember of a request as its state
+class FilterPart : public Part { public: using Part::Part; const char* family() const override { return "filter"; }
+  virtual void forward(StepContext& ctx, const Tensor& u, const Tensor& out) = 0; };
 class FeedForwardPart : public Part { public: using Part::Part; const char* family() const override { return "ffn"; }
   virtual void forward(StepContext& ctx, const Rows& h, const Tensor& x) = 0;
   virtual bool can_store() const { return false; }

@@ -993,6 +993,130 @@ void Ops::gated_head_norm(const Tensor& o, const Tensor& proj, int gate_col, con
   check("recurrent", rc, "gated_head_norm");
 }
 
+// ------------------------------------------------- post-norm layers, short convolutions, differential attention, experts
+void Ops::norm_residual(const Tensor& x, const Tensor& y, const Tensor& gain, float eps, bool accumulate, const int* gather,
+                        int n_gather) {
+  TIMED("norm_residual " + dims(x));
+  const int64_t H = x.ndim == 2 ? x.shape[1] : 0;
+  require(x.ndim == 2 && x.dtype == DType::F32 && x.contiguous() && y.ndim == 2 && y.dtype == DType::F32 && y.contiguous() &&
+              y.shape[1] == H && (gather ? n_gather > 0 : y.shape[0] == x.shape[0]) && gain.dtype == DType::F32 && gain.numel() == H,
+          "norm_residual: x " + x.describe() + ", y " + y.describe() + " or gain " + gain.describe() + " do not fit");
+  int rc = KERNEL("residual", ti_norm_residual)((float*)x.data, (const float*)y.data, (const float*)gain.data, gather, n_gather,
+                                                (int)x.shape[0], (int)H, eps, accumulate ? 1 : 0, (hipStream_t)launch_stream());
+  check("residual", rc, "norm_residual");
+}
+
+void Ops::round_rows(const Tensor& x, const Tensor& out) {
+  TIMED("round_rows " + dims(x));
+  require(x.dtype == DType::F32 && x.contiguous() && out.contiguous() && out.numel() == x.numel(),
+          "round_rows: x " + x.describe() + " and out " + out.describe() + " do not fit");
+  int rc = KERNEL("residual", ti_round_rows)(code(out.dtype, "round_rows"), (const float*)x.data, out.data, (long)x.numel(),
+                                             (hipStream_t)launch_stream());
+  check("residual", rc, "round_rows");
+}
+
+void Ops::scale(const Tensor& x, float s) {
+  TIMED("scale " + dims(x));
+  require(x.dtype == DType::F32 && x.contiguous(), "scale: x " + x.describe() + " must be contiguous float32");
+  int rc = KERNEL("residual", ti_scale)((float*)x.data, s, (long)x.numel(), (hipStream_t)launch_stream());
+  check("residual", rc, "scale");
+}
+
+void Ops::short_conv(const Tensor& u, const Tensor& taps, const Tensor& state, const int* entry_meta, int n_entries,
+                     const int* entry_of, const int* positions, const Tensor& out) {
+  TIMED("short_conv " + dims(u));
+  require(u.ndim == 2 && u.dtype == DType::F32 && u.contiguous() && out.ndim == 2 && out.dtype == DType::F32 && out.contiguous() &&
+              out.shape[0] == u.shape[0] && out.shape[1] == u.shape[1] && out.data != u.data,
+          "short_conv: u " + u.describe() + " and out " + out.describe() + " must be distinct contiguous float32 [M, C]");
+  const int64_t C = u.shape[1];
+  require(taps.ndim == 2 && taps.dtype == DType::F32 && taps.contiguous() && taps.shape[0] == C && taps.shape[1] >= 1,
+          "short_conv: taps " + taps.describe() + " must be float32 [C, taps]");
+  const int64_t K = taps.shape[1];
+  require(K == 1 || (state.defined() && state.dtype == DType::F32 && state.contiguous() && state.ndim == 3 &&
+                     state.shape[1] == K - 1 && state.shape[2] == C),
+          "short_conv: state " + state.describe() + " does not fit [slots, " + std::to_string(K - 1) + ", " + std::to_string(C) + "]");
+  require(entry_meta != nullptr && entry_of != nullptr && positions != nullptr, "short_conv: no entry records");
+  int rc = KERNEL("diff_attention", ti_short_conv)((const float*)u.data, (const float*)taps.data, (float*)state.data, entry_meta,
+                                                   n_entries, entry_of, positions, (float*)out.data, (int)u.shape[0], (int)C, (int)K,
+                                                   (hipStream_t)launch_stream());
+  check("diff_attention", rc, "short_conv");
+}
+
+void Ops::diff_qk_prep(const Tensor& qkv, const float* q_w, const float* k_w, float eps, const Rotation& rot, const int* positions,
+                       const int* slots, const CacheView& view, const Tensor& pool, const Tensor& q_out, int heads, int kv_heads,
+                       int dk, int dv) {
+  TIMED("diff_qk_prep " + dims(qkv));
+  const int64_t M = qkv.shape[0];
+  const int64_t width = (int64_t)heads * 2 * dk + (int64_t)kv_heads * (2 * dk + dv);
+  require(qkv.ndim == 2 && qkv.shape[1] == width && qkv.dtype == DType::F32 && qkv.contiguous(),
+          "diff_qk_prep: qkv " + qkv.describe() + " does not fit [M, " + std::to_string(width) + "] float32");
+  require(q_out.ndim == 2 && q_out.shape[0] == M && q_out.shape[1] == (int64_t)heads * 2 * dk && q_out.contiguous(),
+          "diff_qk_prep: q_out has the wrong shape");
+  check_split_pool("diff_qk_prep", pool, kv_heads, 2 * dk, dv, q_out.dtype);
+  const int rot_dims = rot.inv_freq ? (rot.dims > 0 ? rot.dims : dk) : 0;
+  int rc = KERNEL("diff_attention", ti_diff_qk_prep)(code(q_out.dtype, "diff_qk_prep"), (const float*)qkv.data, q_w, k_w, eps,
+                                                     rot.inv_freq, rot.table, rot.table_len, rot.mag, rot_dims, positions, slots,
+                                                     view.table, view.table_width, pool.data, q_out.data, (int)M, heads, kv_heads, dk,
+                                                     dv, (int)pool.shape[2], (hipStream_t)launch_stream());
+  check("diff_attention", rc, "diff_qk_prep");
+}
+
+void Ops::diff_attention(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
+                         const Tensor& out, int heads, int kv_heads, int dk, int dv, float scale, int block, int window, float lambda,
+                         float eps, float out_scale) {
+  TIMED("diff_attention " + dims(q));
+  const int64_t M = q.shape[0];
+  require(q.ndim == 2 && q.shape[1] == (int64_t)heads * 2 * dk && out.ndim == 2 && out.shape[0] == M &&
+              out.shape[1] == (int64_t)heads * dv && q.dtype == pool.dtype && out.dtype == q.dtype && q.contiguous() && out.contiguous(),
+          "diff_attention: q/out/pool shapes or dtypes do not fit");
+  check_split_pool("diff_attention", pool, kv_heads, 2 * dk, dv, q.dtype);
+  took("[generic]");
+  int rc = KERNEL("diff_attention", ti_diff_attention_rows)(code(q.dtype, "diff_attention"), q.data, pool.data, view.table,
+                                                            view.table_width, positions, slots, out.data, (int)M, heads, kv_heads, dk,
+                                                            dv, (int)pool.shape[2], scale, block, window, lambda, eps, out_scale,
+                                                            (hipStream_t)launch_stream());
+  check("diff_attention", rc, "diff_attention");
+}
+
+void Ops::moe_route(const Tensor& h, const Tensor& router, const Tensor& ids, const Tensor& wts, int top, RouterScore score,
+                    bool renormalize) {
+  TIMED("moe_route " + dims(h) + " experts=" + std::to_string(router.ndim == 2 ? router.shape[0] : 0));
+  require(h.ndim == 2 && h.contiguous() && router.ndim == 2 && router.dtype == DType::F32 && router.contiguous() &&
+              router.shape[1] == h.shape[1],
+          "moe_route: h " + h.describe() + " and router " + router.describe() + " do not fit");
+  const int64_t M = h.shape[0];
+  require(ids.dtype == DType::I32 && ids.contiguous() && ids.numel() == M * top && wts.dtype == DType::F32 && wts.contiguous() &&
+              wts.numel() == M * top,
+          "moe_route: ids and wts must be int32 / float32 [M, top]");
+  int rc = KERNEL("moe", ti_moe_route)(code(h.dtype, "moe_route"), h.data, (const float*)router.data, (int*)ids.data, (float*)wts.data,
+                                       (int)M, (int)h.shape[1], (int)router.shape[0], top, (int)score, renormalize ? 1 : 0,
+                                       (hipStream_t)launch_stream());
+  check("moe", rc, "moe_route");
+}
+
+void Ops::moe_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, const Tensor& up, const Tensor& down, const Tensor& y,
+                      int experts, bool scale_input) {
+  TIMED("moe_experts " + dims(h) + " * " + dims(up));
+  require(h.ndim == 2 && h.contiguous() && up.ndim == 2 && down.ndim == 2 && up.contiguous() && down.contiguous() &&
+              up.dtype == h.dtype && down.dtype == h.dtype && experts > 0,
+          "moe_experts: h, up and down must be matrices of one dtype");
+  const int64_t M = h.shape[0], W = h.shape[1];
+  require(up.shape[1] == W && up.shape[0] % experts == 0, "moe_experts: up " + up.describe() + " does not fit");
+  const int64_t F = up.shape[0] / experts;
+  require(down.shape[0] == (int64_t)experts * W && down.shape[1] == F, "moe_experts: down " + down.describe() + " does not fit");
+  require(y.ndim == 2 && y.dtype == DType::F32 && y.contiguous() && y.shape[0] == M && y.shape[1] == W,
+          "moe_experts: y " + y.describe() + " does not fit");
+  require(ids.dtype == DType::I32 && wts.dtype == DType::F32 && ids.numel() == wts.numel() && (M == 0 || ids.numel() % M == 0),
+          "moe_experts: ids and wts must be int32 / float32 [M, top]");
+  if (M == 0) return;
+  const int top = (int)(ids.numel() / M);
+  took("[rows]");
+  int rc = KERNEL("moe", ti_moe_experts_rows)(code(h.dtype, "moe_experts"), h.data, (const int*)ids.data, (const float*)wts.data,
+                                              up.data, down.data, (float*)y.data, (int)M, (int)W, (int)F, top, scale_input ? 1 : 0,
+                                              (hipStream_t)launch_stream());
+  check("moe", rc, "moe_experts");
+}
+
 // ----------------------------------------------------------------------------------- sampling
 void Ops::argmax(const Tensor& logits, int* out) {
   TIMED("argmax " + dims(logits));

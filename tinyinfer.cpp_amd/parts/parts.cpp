@@ -28,9 +28,19 @@
 //   block     "parallel"    x += s1 * mixer(norm(x)) + s2 * ffn(norm(x)) with learned per-channel scales
 //   block     "add_vector"  x += a row of a learned table (what a looped run of layers adds before each pass)
 //
+//   norm      "rmsnorm" with `one_plus`: the checkpoint holds the gain minus one; the norm onto the residual (forward_add)
+//   embedding "table" with `norm`: a norm of the looked-up rows, in 32-bit, in place
+//   pos       "rope_partial" rotation of the first `dims` entries of a head, frequencies interpolated between the plain
+//                           ones and the ones divided by `factor` (YaRN), cosine and sine times 0.1 ln(factor) + 1
+//   filter    "short_conv"  a causal convolution of a few taps over time on every channel, the last taps - 1 rows as state
+//   mixer     "diff_attention" two softmax maps a head over one value, subtracted, normed; keys visible per block
+//   ffn       "moe"         routed experts with sigmoid or softmax scores on the experts' inputs or outputs
+//   block     "post_norm"   x += norm1(mixer(x)); x += norm2(ffn(x)): the sublayers read x itself
+//
 // A part gets every size and constant as a parameter and never looks at the model it sits in.
 #include <algorithm>
 #include <cmath>
+#include <cstring>
 #include <mutex>
 
 #include "../include/inference.h"
@@ -66,7 +76,7 @@ std::map<std::pair<std::string, std::string>, Registered>& table() {
   static std::map<std::pair<std::string, std::string>, Registered> t;
   return t;
 }
-const char* FAMILIES[] = {"embedding", "norm", "pos", "mixer", "ffn", "block", "head"};
+const char* FAMILIES[] = {"embedding", "norm", "pos", "mixer", "ffn", "block", "head", "filter"};
 void register_builtin_parts();
 void ensure_builtins() {
   static std::once_flag once;
@@ -91,6 +101,9 @@ std::string tensor_name(const Json& p, const char* key, const std::string& prefi
 }
 }  // namespace
 
+void NormPart::forward_add(StepContext&, const Tensor&, const Tensor&, bool, const int*, int) {
+  throw EngineError(std::string("the norm '") + kind_name() + "' cannot write into the residual");
+}
 void MixerPart::forward_store(StepContext&, const Rows&, const Tensor&) {
   throw EngineError(std::string("the mixer '") + kind_name() + "' cannot write its output apart from the residual");
 }
@@ -169,6 +182,10 @@ class Embedding final : public EmbeddingPart {
       if (c.first == "pos") pos = std::dynamic_pointer_cast<PositionPart>(c.second);
     if (!pos && p.has("pos")) pos = std::dynamic_pointer_cast<PositionPart>(build_part("pos", PartSpec::from_json(p.at("pos")), prefix));
     if (pos && !pos->additive()) throw ConfigError("embedding: the position encoding '" + std::string(pos->kind_name()) + "' is not additive");
+    for (const auto& c : children)
+      if (c.first == "norm") norm = std::dynamic_pointer_cast<NormPart>(c.second);
+    if (!norm && p.has("norm")) norm = std::dynamic_pointer_cast<NormPart>(build_part("norm", PartSpec::from_json(p.at("norm")), prefix));
+    if (norm && !norm->can_add()) throw ConfigError("embedding: the norm '" + std::string(norm->kind_name()) + "' cannot write 32-bit rows");
   }
   const char* kind_name() const override { return "table"; }
   std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
@@ -177,32 +194,39 @@ class Embedding final : public EmbeddingPart {
     return {{name, n}};
   }
   std::vector<std::shared_ptr<Part>> children() const override {
-    if (pos) return {pos};
-    return {};
+    std::vector<std::shared_ptr<Part>> v;
+    if (pos) v.push_back(pos);
+    if (norm) v.push_back(norm);
+    return v;
   }
   std::vector<std::string> child_slots() const override {
-    if (pos) return {"pos"};
-    return {};
+    std::vector<std::string> v;
+    if (pos) v.push_back("pos");
+    if (norm) v.push_back("norm");
+    return v;
   }
   void load(WeightSource& src) override { weight = src.fetch(name, tensors()[0].second); }
   void forward(StepContext& ctx, const Tensor& x) override {
     ctx.ops.embed(weight, ctx.tokens, ctx.M, x, ctx.fed_tokens, ctx.n_fed_tokens);
     if (pos) pos->add(ctx, x);
+    if (norm) norm->forward_add(ctx, x, x, false);
   }
   bool reads_through_ops() const override { return true; }
   std::vector<std::pair<std::string, Tensor>> held() const override { return {{"weight", weight}}; }
   int64_t vocab, dim;
   std::string name;
   std::shared_ptr<PositionPart> pos;
+  std::shared_ptr<NormPart> norm;      // `norm`: applied to the looked-up rows (after `pos`), in 32-bit
   Tensor weight;
 };
 
+// `scale`: the logits are multiplied by it.
 // `tied`: 1 reads `tied_to`; 0 reads its own `weight`; -1 takes its own weight if the checkpoint
 // holds one and `tied_to` otherwise.
 class LMHead final : public HeadPart {
  public:
-  LMHead(const std::string& prefix, int64_t vocab, int64_t dim, int tied, std::string tied_to, std::string own_name)
-      : HeadPart(prefix), vocab(vocab), dim(dim), tied(tied), tied_to(std::move(tied_to)), own_name(std::move(own_name)) {}
+  LMHead(const std::string& prefix, int64_t vocab, int64_t dim, int tied, std::string tied_to, std::string own_name, double scale = 1.0)
+      : HeadPart(prefix), vocab(vocab), dim(dim), tied(tied), tied_to(std::move(tied_to)), own_name(std::move(own_name)), scale((float)scale) {}
   const char* kind_name() const override { return "linear"; }
   std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
     TensorNeed must, may;
@@ -224,6 +248,7 @@ class LMHead final : public HeadPart {
     const Tensor& rows = h.materialize(ctx.ops);
     Tensor logits = ctx.buf("head.logits", DType::F32, {rows.shape[0], vocab});
     ctx.ops.linear(rows, weight, logits, Ops::Store);
+    if (scale != 1.f) ctx.ops.scale(logits, scale);
     return logits;
   }
   bool reads_through_ops() const override { return true; }
@@ -231,6 +256,7 @@ class LMHead final : public HeadPart {
   int64_t vocab, dim;
   int tied;
   std::string tied_to, own_name;
+  float scale;                 // `scale`: a factor on the logits
   Tensor weight;
 };
 
@@ -239,8 +265,9 @@ class LMHead final : public HeadPart {
 // the weight's name in the checkpoint (default: prefix + ".weight").
 class RMSNorm final : public NormPart {
  public:
-  RMSNorm(const std::string& prefix, int64_t dim, double eps, bool scalar = false, std::string name_ = "")
-      : NormPart(prefix), dim(dim), eps((float)eps), scalar(scalar), name(name_.empty() ? join(prefix, "weight") : std::move(name_)) {}
+  RMSNorm(const std::string& prefix, int64_t dim, double eps, bool scalar = false, std::string name_ = "", bool one_plus = false)
+      : NormPart(prefix), dim(dim), eps((float)eps), scalar(scalar), one_plus(one_plus),
+        name(name_.empty() ? join(prefix, "weight") : std::move(name_)) {}
   const char* kind_name() const override { return "rmsnorm"; }
   bool can_be_lazy() const override { return true; }
   bool reads_through_ops() const override { return true; }
@@ -248,11 +275,25 @@ class RMSNorm final : public NormPart {
     TensorNeed n;
     if (!scalar) n.shape = {dim};
     n.role = TensorNeed::Vector;
-    n.a = 1.0;
+    n.a = one_plus ? 0.0 : 1.0;
     n.b = 0.1;
     return {{name, n}};
   }
   void load(WeightSource& src) override {
+    if (one_plus) {
+      // the gain is 1 + w, formed once in 32-bit (the stored tensor may serve another part as it is)
+      const Tensor stored = src.fetch(name, tensors()[0].second);
+      if (scalar) {
+        const Tensor one = src.alloc(DType::F32, {1});
+        plus_one(stored, one, src.to_host);
+        weight = src.alloc(DType::F32, {dim});
+        spread(one, weight, src.to_host);
+      } else {
+        weight = src.alloc(DType::F32, {dim});
+        plus_one(stored, weight, src.to_host);
+      }
+      return;
+    }
     if (!scalar) {
       weight = src.fetch(name, tensors()[0].second);
       return;
@@ -262,6 +303,11 @@ class RMSNorm final : public NormPart {
     spread(one, weight, src.to_host);
   }
   static void spread(const Tensor& one, const Tensor& all, bool on_host);     // all[:] = one[0]
+  static void plus_one(const Tensor& w, const Tensor& out, bool on_host);     // out = 1 + w
+  bool can_add() const override { return true; }
+  void forward_add(StepContext& ctx, const Tensor& y, const Tensor& x, bool accumulate, const int* gather, int n_gather) override {
+    ctx.ops.norm_residual(x, y, weight, eps, accumulate, gather, n_gather);
+  }
   // x: f32 [M, dim].  With `rows` only those rows of x are read, in that order.  `lazy`: the
   // consumer feeds the result to one product and nothing else, so where a kernel can take the
   // norm in, the rows come back not yet computed.
@@ -282,7 +328,7 @@ class RMSNorm final : public NormPart {
   std::vector<std::pair<std::string, Tensor>> held() const override { return {{"weight", weight}}; }
   int64_t dim;
   float eps;
-  bool scalar;
+  bool scalar, one_plus;     // one_plus: the checkpoint holds the gain minus one (weights kept around zero)
   std::string name;
   Tensor weight;
 };
@@ -1074,7 +1120,476 @@ class AddVectorBlock final : public BlockPart {
   Tensor table;
 };
 
+// Rotation of the first `dims` entries of a head in the half-split layout (entry i turns with entry i + dims / 2 by
+// the angle pos * f_i, f_i = base^(-2i / dims)); the rest of the head passes.  `scaling` {factor, original, fast, slow}
+// interpolates the frequencies as YaRN does: with dim(t) = dims ln(original / (2 pi t)) / (2 ln base),
+// lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), dims - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1),
+// the frequency is f_i / factor * ramp_i + f_i (1 - ramp_i), and cosine and sine are multiplied by 0.1 ln(factor) + 1.
+// Frequencies and, for the positions an engine serves, cosines and sines are built on the host in double precision
+// and rounded once; a table is immutable and lives as long as the part (captured graphs hold its address).
+class RotaryPartial final : public PositionPart {
+ public:
+  RotaryPartial(const std::string& prefix, const Json& p) : PositionPart(prefix) {
+    dims = (int)param_int(p, "dims");
+    base = param_float(p, "base");
+    if (dims < 0 || dims % 2) throw ConfigError("rotary: " + std::to_string(dims) + " rotated entries: must be even and not negative");
+    if (!(base > 0.0)) throw ConfigError("rotary: base must be positive");
+    if (p.has("scaling")) {
+      const Json& sc = p.at("scaling");
+      factor = param_float(sc, "factor");
+      original = param_float(sc, "original");
+      fast = param_float(sc, "fast");
+      slow = param_float(sc, "slow");
+      if (!(factor > 0.0) || !(original > 0.0) || !(fast > 0.0) || !(slow > 0.0))
+        throw ConfigError("rotary: scaling factor, original, fast and slow must be positive");
+      scaled = true;
+    }
+    const int half = dims / 2;
+    freq.resize(half);
+    for (int i = 0; i < half; ++i) freq[i] = std::pow(base, -2.0 * i / dims);
+    if (scaled) {
+      const double pi = 3.14159265358979323846;
+      auto dim_of = [&](double turns) { return dims * std::log(original / (2.0 * pi * turns)) / (2.0 * std::log(base)); };
+      const double lo = std::max(std::floor(dim_of(fast)), 0.0);
+      const double hi = std::min(std::ceil(dim_of(slow)), (double)(dims - 1));
+      for (int i = 0; i < half; ++i) {
+        const double ramp = std::min(1.0, std::max(0.0, (i - lo) / std::max(hi - lo, 0.001)));
+        freq[i] = freq[i] / factor * ramp + freq[i] * (1.0 - ramp);
+      }
+      mag = 0.1 * std::log(factor) + 1.0;
+    }
+  }
+  const char* kind_name() const override { return "rope_partial"; }
+  void prepare(Ops&, int max_seq) override {
+    std::lock_guard<std::mutex> lock(g_rope_mutex);
+    const int half = dims / 2;
+    if (half == 0) return;
+    if (!inv_freq.data()) {
+      std::vector<float> f32(freq.begin(), freq.end());
+      inv_freq = DeviceBuffer((size_t)half * 4);
+      RotaryNeox::upload(inv_freq.data(), f32.data(), (size_t)half * 4);
+    }
+    if (max_seq <= table_len) return;
+    std::vector<float> host((size_t)max_seq * half * 2);
+    for (int p = 0; p < max_seq; ++p)
+      for (int i = 0; i < half; ++i) {
+        const double a = (double)p * freq[i];
+        host[((size_t)p * half + i) * 2] = (float)(std::cos(a) * mag);
+        host[((size_t)p * half + i) * 2 + 1] = (float)(std::sin(a) * mag);
+      }
+    tables.emplace_back(host.size() * 4);
+    RotaryNeox::upload(tables.back().data(), host.data(), host.size() * 4);
+    table_len = max_seq;
+  }
+  bool fused(Ops::Rotation& rot) const override {
+    std::lock_guard<std::mutex> lock(g_rope_mutex);
+    if (dims == 0 || !inv_freq.data()) return false;
+    rot.inv_freq = (const float*)inv_freq.data();
+    rot.table = tables.empty() ? nullptr : (const float*)tables.back().data();
+    rot.table_len = table_len;
+    rot.dims = dims;
+    rot.mag = (float)mag;
+    return true;
+  }
+  void apply(StepContext&, const Tensor&, const Tensor&) override {
+    throw EngineError("the partial rotation is applied by the kernels that prepare queries and keys (fused)");
+  }
+  std::vector<std::pair<std::string, Tensor>> held() const override {
+    if (!inv_freq.data()) return {};
+    std::vector<std::pair<std::string, Tensor>> h = {{"inv_freq", Tensor(inv_freq.data(), DType::F32, {dims / 2})}};
+    if (table_len) h.emplace_back("table", Tensor(tables.back().data(), DType::F32, {table_len, dims / 2, 2}));
+    return h;
+  }
+  int dims = 0;
+  double base = 10000.0, factor = 1.0, original = 0.0, fast = 0.0, slow = 0.0, mag = 1.0;
+  bool scaled = false;
+  std::vector<double> freq;
+  DeviceBuffer inv_freq;
+  std::vector<DeviceBuffer> tables;     // oldest first; the last one is read
+  int table_len = 0;
+};
+
+// A causal convolution over time on every channel of the rows it is given: y_t = sum_j w[:, j] u_(t - taps + 1 + j), zeros
+// before a sequence's start, no bias.  `segments`: [[tensor name, channels], ...], the taps [channels, taps] of runs of
+// channels side by side (the parts of a fused projection each bring their own tensor).  The last taps - 1 rows of every
+// request are its state (32-bit, zeroed at admission: the zeros before the start).
+class ShortConv final : public FilterPart {
+ public:
+  ShortConv(const std::string& prefix, const Json& p) : FilterPart(prefix) {
+    taps = (int)param_int(p, "taps");
+    if (taps < 1) throw ConfigError("short_conv: taps must be at least 1");
+    const Json* seg = p.find("segments");
+    if (!seg || seg->type() != Json::Array || seg->size() == 0) throw ConfigError("short_conv: 'segments' must list [tensor, channels] pairs");
+    for (const Json& s : seg->items()) {
+      if (s.type() != Json::Array || s.size() != 2 || s[0].type() != Json::String || !s[1].is_number() || s[1].as_int() <= 0)
+        throw ConfigError("short_conv: a segment is [tensor name, channels]");
+      segments.emplace_back(s[0].as_string(), s[1].as_int());
+      channels += s[1].as_int();
+    }
+  }
+  const char* kind_name() const override { return "short_conv"; }
+  bool reads_through_ops() const override { return true; }
+  std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
+    std::vector<std::pair<std::string, TensorNeed>> t;
+    for (const auto& s : segments) {
+      TensorNeed n;
+      n.shape = {s.second, (int64_t)taps};
+      n.role = TensorNeed::Vector;
+      n.a = 1.0 / taps;
+      n.b = 0.3;
+      t.emplace_back(s.first, n);
+    }
+    return t;
+  }
+  void load(WeightSource& src) override {
+    w = src.alloc(DType::F32, {channels, (int64_t)taps});
+    int64_t at = 0;
+    for (const auto& s : segments) {
+      src.fill(s.first, w.rows(at, s.second));
+      at += s.second;
+    }
+  }
+  bool has_cache() const override { return taps > 1; }
+  CacheNeed cache_need() const override {
+    CacheNeed n;
+    n.kind = CacheNeed::State;
+    n.state_shape = {(int64_t)taps - 1, channels};
+    return n;
+  }
+  void forward(StepContext& ctx, const Tensor& u, const Tensor& out) override {
+    Tensor state;
+    if (taps > 1) {
+      const auto bound = ctx.binding(this);
+      state = ctx.state(bound.first, bound.second);
+    }
+    ctx.ops.short_conv(u, w, state, ctx.entry_meta, (int)ctx.entries.size(), ctx.slots, ctx.positions, out);
+  }
+  std::vector<std::pair<std::string, Tensor>> held() const override { return {{"w", w}}; }
+  int taps = 1;
+  int64_t channels = 0;
+  std::vector<std::pair<std::string, int64_t>> segments;
+  Tensor w;
+};
+
+// Differential attention.  Every one of the `heads` query heads holds two maps: q has heads x 2 x head_dim rows, k has
+// kv_heads x 2 x head_dim (head by head as [map 1, map 2]), v has kv_heads x v_head_dim; query head h reads key/value
+// head floor(h / (heads / kv_heads)).  Behind the fused projection: the child `conv` (a filter over time, optional) on all
+// its channels, then per head and map an RMS norm over head_dim (weights `q_norm`, `k_norm` of size head_dim, shared by
+// all heads and maps; `qk_norm` false: none) and the rotation of the child `pos` (optional); v is left alone.  Each map is
+// a softmax attention of its own, scores (q . k) * scale over the keys that are not later and lie in the query's block of
+// `block` positions counted from 0 (0: no blocks; `window` likewise optional); both read the same values.  With a1, a2 the
+// maps' outputs and lambda = exp(sum(lq1 * lk1)) - exp(sum(lq2 * lk2)) + diff (vectors of size head_dim, one number a
+// layer, formed once when the weights load): o = a1 - lambda a2, divided by its root mean square over v_head_dim (eps, no
+// weight), times 1 - diff; then the output projection.  Scores, softmax, lambda and the norms are 32-bit.
+class DiffAttention final : public MixerPart {
+ public:
+  DiffAttention(const std::string& prefix, const Json& p, const PartChildren& children) : MixerPart(prefix) {
+    hidden = param_int(p, "hidden");
+    heads = (int)param_int(p, "heads");
+    kv_heads = p.has("kv_heads") ? (int)param_int(p, "kv_heads") : heads;
+    dk = (int)param_int(p, "head_dim");
+    dv = p.has("v_head_dim") ? (int)param_int(p, "v_head_dim") : dk;
+    if (heads <= 0 || kv_heads <= 0 || heads % kv_heads)
+      throw ConfigError("diff_attention: heads " + std::to_string(heads) + " not a multiple of kv_heads " + std::to_string(kv_heads));
+    if (dk < 1 || dk > 256 || dv < 1 || dv > 256)
+      throw ConfigError("diff_attention: key size " + std::to_string(dk) + " / value size " + std::to_string(dv) + " are not served (up to 256)");
+    diff = param_float(p, "diff");
+    eps = (float)(p.has("eps") ? param_float(p, "eps") : 1e-6);
+    scale = p.has("scale") ? (float)param_float(p, "scale") : (float)(1.0 / std::sqrt((double)dk));
+    block = p.has("block") ? (int)param_int(p, "block") : 0;
+    window = p.has("window") ? (int)param_int(p, "window") : 0;
+    if (block < 0 || window < 0) throw ConfigError("diff_attention: block and window must not be negative");
+    qk_norm = p.has("qk_norm") ? p.at("qk_norm").as_bool() : true;
+    for (const auto& c : children) {
+      if (c.first == "pos") pos = std::dynamic_pointer_cast<PositionPart>(c.second);
+      if (c.first == "conv") conv = std::dynamic_pointer_cast<FilterPart>(c.second);
+    }
+    if (!pos && p.has("pos")) pos = std::dynamic_pointer_cast<PositionPart>(build_part("pos", PartSpec::from_json(p.at("pos")), prefix));
+    if (!conv && p.has("conv")) conv = std::dynamic_pointer_cast<FilterPart>(build_part("filter", PartSpec::from_json(p.at("conv")), prefix));
+    nq = (int64_t)heads * 2 * dk;
+    nk = (int64_t)kv_heads * 2 * dk;
+    nv = (int64_t)kv_heads * dv;
+    no = (int64_t)heads * dv;
+    n_q = tensor_name(p, "q", prefix, "q");
+    n_k = tensor_name(p, "k", prefix, "k");
+    n_v = tensor_name(p, "v", prefix, "v");
+    n_o = tensor_name(p, "o", prefix, "o");
+    n_qn = tensor_name(p, "q_norm", prefix, "q.norm");
+    n_kn = tensor_name(p, "k_norm", prefix, "k.norm");
+    for (int i = 0; i < 4; ++i) {
+      static const char* keys[4] = {"lq1", "lk1", "lq2", "lk2"};
+      n_l[i] = tensor_name(p, keys[i], prefix, keys[i]);
+    }
+  }
+  const char* kind_name() const override { return "diff_attention"; }
+  bool can_store() const override { return true; }
+  bool takes_lazy_norm() const override { return true; }
+  bool reads_through_ops() const override { return true; }
+  std::vector<std::shared_ptr<Part>> children() const override {
+    std::vector<std::shared_ptr<Part>> v;
+    if (pos) v.push_back(pos);
+    if (conv) v.push_back(conv);
+    return v;
+  }
+  std::vector<std::string> child_slots() const override {
+    std::vector<std::string> v;
+    if (pos) v.push_back("pos");
+    if (conv) v.push_back("conv");
+    return v;
+  }
+  TensorNeed vector_need(double a, double b) const {
+    TensorNeed n;
+    n.shape = {dk};
+    n.role = TensorNeed::Vector;
+    n.a = a;
+    n.b = b;
+    return n;
+  }
+  std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
+    std::vector<std::pair<std::string, TensorNeed>> t;
+    TensorNeed q, k, v, o;
+    q.shape = {nq, hidden};
+    k.shape = {nk, hidden};
+    v.shape = {nv, hidden};
+    o.shape = {hidden, no};
+    t.emplace_back(n_q, q);
+    t.emplace_back(n_k, k);
+    t.emplace_back(n_v, v);
+    t.emplace_back(n_o, o);
+    if (qk_norm) {
+      t.emplace_back(n_qn, vector_need(1.0, 0.1));
+      t.emplace_back(n_kn, vector_need(1.0, 0.1));
+    }
+    for (int i = 0; i < 4; ++i) t.emplace_back(n_l[i], vector_need(0.0, 0.1));
+    return t;
+  }
+  void load(WeightSource& src) override {
+    w_qkv = src.alloc(src.matrix_dtype, {nq + nk + nv, hidden});
+    src.fill(n_q, w_qkv.rows(0, nq));
+    src.fill(n_k, w_qkv.rows(nq, nk));
+    src.fill(n_v, w_qkv.rows(nq + nk, nv));
+    TensorNeed o;
+    o.shape = {hidden, no};
+    w_o = src.fetch(n_o, o);
+    if (qk_norm) {
+      q_norm_w = src.fetch(n_qn, vector_need(1.0, 0.1));
+      k_norm_w = src.fetch(n_kn, vector_need(1.0, 0.1));
+    }
+    Tensor l[4];
+    for (int i = 0; i < 4; ++i) l[i] = src.fetch(n_l[i], vector_need(0.0, 0.1));
+    lambda = lambda_of(l, dk, diff, src.to_host);
+  }
+  // exp(sum(lq1 * lk1)) - exp(sum(lq2 * lk2)) + diff, sums and exponentials in 32-bit
+  static float lambda_of(const Tensor l[4], int dk, double diff, bool on_host);
+  bool has_cache() const override { return true; }
+  CacheNeed cache_need() const override {
+    CacheNeed n;
+    n.kind = CacheNeed::PagedKV;
+    n.kv_heads = kv_heads;
+    n.head_dim = 2 * dk;          // a row's two maps side by side
+    n.v_dim = dv != 2 * dk ? dv : 0;
+    n.window = window;
+    n.block = block;
+    return n;
+  }
+  void run(StepContext& ctx, const Rows& h, const Tensor& out, Ops::Epilogue epi) {
+    const int64_t M = h.t.shape[0];
+    const int64_t width = nq + nk + nv;
+    Tensor qkv = ctx.buf("dattn.qkv", DType::F32, {M, width});
+    ctx.ops.linear(h, w_qkv, qkv, Ops::Store);
+    if (conv) {
+      Tensor mixed = ctx.buf("dattn.conv", DType::F32, {M, width});
+      conv->forward(ctx, qkv, mixed);
+      qkv = mixed;
+    }
+    const auto bound = ctx.binding(this);
+    const Tensor pool = ctx.kv_pool(bound.first, bound.second);
+    const Ops::CacheView view = ctx.cache_view(bound.first);
+    Ops::Rotation rot;
+    if (pos && !pos->fused(rot)) throw EngineError("diff_attention: the position encoding '" + std::string(pos->kind_name()) + "' has no fused form");
+    Tensor q = ctx.buf("dattn.q", ctx.act_dtype, {M, nq});
+    ctx.ops.diff_qk_prep(qkv, q_norm_w.ptr<float>(), k_norm_w.ptr<float>(), eps, rot, ctx.positions, ctx.slots, view, pool, q, heads,
+                         kv_heads, dk, dv);
+    Tensor a = ctx.buf("dattn.out", ctx.act_dtype, {M, no});
+    ctx.ops.diff_attention(q, pool, view, ctx.positions, ctx.slots, a, heads, kv_heads, dk, dv, scale, block, window, lambda, eps,
+                           (float)(1.0 - diff));
+    ctx.ops.linear(a, w_o, out, epi, false);
+  }
+  void forward(StepContext& ctx, const Rows& h, const Tensor& x) override { run(ctx, h, x, Ops::Add); }
+  void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override { run(ctx, h, y, Ops::Store); }
+  std::vector<std::pair<std::string, Tensor>> held() const override {
+    return {{"w_qkv", w_qkv}, {"w_o", w_o}, {"q_norm_w", q_norm_w}, {"k_norm_w", k_norm_w}};
+  }
+  int64_t hidden = 0, nq = 0, nk = 0, nv = 0, no = 0;
+  int heads = 0, kv_heads = 0, dk = 0, dv = 0, block = 0, window = 0;
+  bool qk_norm = true;
+  double diff = 0.0;
+  float eps = 1e-6f, scale = 1.f, lambda = 0.f;
+  std::string n_q, n_k, n_v, n_o, n_qn, n_kn, n_l[4];
+  std::shared_ptr<PositionPart> pos;
+  std::shared_ptr<FilterPart> conv;
+  Tensor w_qkv, w_o, q_norm_w, k_norm_w;
+};
+
+// A mixture of experts: `experts` small feed-forward layers W_down act(W_up h) without biases (tensors prefix + ".e<i>.up"
+// [intermediate, hidden], ".e<i>.down"), of which each token uses the `top` with the largest scores.  Router logits
+// W_router h and the scores (`score`: "sigmoid", or "softmax" over all experts) are 32-bit; `renormalize`: the chosen
+// scores are divided by their sum.  `scale_input` true: the score multiplies the expert's input, the output is
+// sum_e expert_e(s_e h); false: its output.  `activation`: "relu2", the square of relu.
+class MoE final : public FeedForwardPart {
+ public:
+  MoE(const std::string& prefix, const Json& p) : FeedForwardPart(prefix) {
+    hidden = param_int(p, "hidden");
+    intermediate = param_int(p, "intermediate");
+    experts = (int)param_int(p, "experts");
+    top = (int)param_int(p, "top");
+    if (hidden <= 0 || intermediate <= 0) throw ConfigError("moe: sizes must be positive");
+    if (experts < 1 || experts > 1024) throw ConfigError("moe: " + std::to_string(experts) + " experts are not served (1 to 1024)");
+    if (top < 1 || top > experts || top > 64)
+      throw ConfigError("moe: top " + std::to_string(top) + " must lie between 1 and the number of experts (and at most 64)");
+    if ((hidden + intermediate) * 4 > 64 * 1024)
+      throw ConfigError("moe: a width of " + std::to_string(hidden) + " beside an expert size of " + std::to_string(intermediate) +
+                        " is not served (the rows of one token and expert must fit 64 KB)");
+    const std::string act = p.has("activation") ? p.at("activation").as_string() : "relu2";
+    if (act != "relu2") throw ConfigError("moe: activation '" + act + "' is not served (only 'relu2')");
+    const std::string sc = p.has("score") ? p.at("score").as_string() : "sigmoid";
+    if (sc != "sigmoid" && sc != "softmax") throw ConfigError("moe: score '" + sc + "' is not served (sigmoid, softmax)");
+    score = sc == "softmax" ? Ops::Softmax : Ops::Sigmoid;
+    renormalize = p.has("renormalize") && p.at("renormalize").as_bool();
+    scale_input = !p.has("scale_input") || p.at("scale_input").as_bool();
+    n_router = tensor_name(p, "router", prefix, "router");
+  }
+  const char* kind_name() const override { return "moe"; }
+  bool reads_through_ops() const override { return true; }
+  bool can_store() const override { return true; }
+  std::string expert_name(int e, const char* t) const { return join(prefix, "e" + std::to_string(e) + "." + t); }
+  std::vector<std::pair<std::string, TensorNeed>> tensors() const override {
+    std::vector<std::pair<std::string, TensorNeed>> t;
+    TensorNeed up, down, router;
+    up.shape = {intermediate, hidden};
+    down.shape = {hidden, intermediate};
+    router.shape = {(int64_t)experts, hidden};
+    router.role = TensorNeed::Vector;      // held in 32-bit whatever the engine's dtype
+    router.b = 0.1;
+    for (int e = 0; e < experts; ++e) {
+      t.emplace_back(expert_name(e, "up"), up);
+      t.emplace_back(expert_name(e, "down"), down);
+    }
+    t.emplace_back(n_router, router);
+    return t;
+  }
+  void load(WeightSource& src) override {
+    // the experts' matrices one under the other: a kernel finds expert e at row e * its rows
+    w_up = src.alloc(src.matrix_dtype, {(int64_t)experts * intermediate, hidden});
+    w_down = src.alloc(src.matrix_dtype, {(int64_t)experts * hidden, intermediate});
+    for (int e = 0; e < experts; ++e) {
+      src.fill(expert_name(e, "up"), w_up.rows((int64_t)e * intermediate, intermediate));
+      src.fill(expert_name(e, "down"), w_down.rows((int64_t)e * hidden, hidden));
+    }
+    TensorNeed router;
+    router.shape = {(int64_t)experts, hidden};
+    router.role = TensorNeed::Vector;
+    w_router = src.fetch(n_router, router);
+  }
+  void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override {
+    const Tensor& rows = h.materialize(ctx.ops);
+    const int64_t M = rows.shape[0];
+    Tensor ids = ctx.buf("moe.ids", DType::I32, {M, (int64_t)top});
+    Tensor wts = ctx.buf("moe.wts", DType::F32, {M, (int64_t)top});
+    ctx.ops.moe_route(rows, w_router, ids, wts, top, score, renormalize);
+    ctx.ops.moe_experts(rows, ids, wts, w_up, w_down, y, experts, scale_input);
+  }
+  void forward(StepContext& ctx, const Rows& h, const Tensor& x) override {
+    Tensor y = ctx.buf("moe.y", DType::F32, {x.shape[0], hidden});
+    forward_store(ctx, h, y);
+    ctx.ops.scaled_add(x, y, Tensor(), Tensor(), Tensor());
+  }
+  std::vector<std::pair<std::string, Tensor>> held() const override { return {{"w_up", w_up}, {"w_down", w_down}, {"w_router", w_router}}; }
+  int64_t hidden = 0, intermediate = 0;
+  int experts = 0, top = 0;
+  Ops::RouterScore score = Ops::Sigmoid;
+  bool renormalize = false, scale_input = true;
+  std::string n_router;
+  Tensor w_up, w_down, w_router;
+};
+
+// x += norm1(mixer(x)); x += norm2(ffn(x)).  The sublayers read the residual itself (rounded to the compute dtype where
+// that is not 32-bit) and the norms are taken on what they return, in 32-bit, straight into the residual.  A layer may
+// have no feed-forward (then no norm2 either).
+class PostNormBlock final : public BlockPart {
+ public:
+  PostNormBlock(const std::string& prefix, const PartChildren& c) : BlockPart(prefix) {
+    for (const auto& kv : c) {
+      if (kv.first == "norm1") norm1 = std::dynamic_pointer_cast<NormPart>(kv.second);
+      if (kv.first == "mixer") mixer = std::dynamic_pointer_cast<MixerPart>(kv.second);
+      if (kv.first == "norm2") norm2 = std::dynamic_pointer_cast<NormPart>(kv.second);
+      if (kv.first == "ffn") ffn = std::dynamic_pointer_cast<FeedForwardPart>(kv.second);
+    }
+    if (!norm1 || !mixer) throw ConfigError("block 'post_norm' needs norm1 and mixer parts (norm2 and ffn are optional)");
+    if ((ffn != nullptr) != (norm2 != nullptr)) throw ConfigError("block 'post_norm': norm2 and ffn come together or not at all");
+    if (!norm1->can_add() || (norm2 && !norm2->can_add())) throw ConfigError("block 'post_norm': its norms must be able to write into the residual");
+    if (!mixer->can_store() || (ffn && !ffn->can_store()))
+      throw ConfigError("block 'post_norm': its mixer and feed-forward must be able to write their output apart from the residual");
+  }
+  const char* kind_name() const override { return "post_norm"; }
+  bool reads_through_ops() const override { return true; }
+  std::vector<std::shared_ptr<Part>> children() const override {
+    std::vector<std::shared_ptr<Part>> v = {norm1, mixer};
+    if (ffn) {
+      v.push_back(norm2);
+      v.push_back(ffn);
+    }
+    return v;
+  }
+  std::vector<std::string> child_slots() const override {
+    std::vector<std::string> v = {"norm1", "mixer"};
+    if (ffn) {
+      v.push_back("norm2");
+      v.push_back("ffn");
+    }
+    return v;
+  }
+  // the rows a sublayer reads: the residual itself in a 32-bit engine, else its rounding
+  Rows input(StepContext& ctx, const Tensor& x) {
+    ctx.ops.flush();
+    Rows h;
+    if (ctx.act_dtype == DType::F32) {
+      h.t = x;
+      return h;
+    }
+    h.t = ctx.buf("post_norm.h", ctx.act_dtype, {x.shape[0], x.shape[1]});
+    ctx.ops.round_rows(x, h.t);
+    return h;
+  }
+  void forward(StepContext& ctx, const Tensor& x) override {
+    Tensor y = ctx.buf("post_norm.y", DType::F32, {x.shape[0], x.shape[1]});
+    mixer->forward_store(ctx, input(ctx, x), y);
+    norm1->forward_add(ctx, y, x, true);
+    if (!ffn) return;
+    ffn->forward_store(ctx, input(ctx, x), y);
+    norm2->forward_add(ctx, y, x, true);
+  }
+  std::shared_ptr<NormPart> norm1, norm2;
+  std::shared_ptr<MixerPart> mixer;
+  std::shared_ptr<FeedForwardPart> ffn;
+};
+
 void register_builtin_parts() {
+  register_part("pos", "rope_partial", [](const std::string& prefix, const Json& p, const PartChildren&) {
+    return std::make_shared<RotaryPartial>(prefix, p);
+  });
+  register_part("filter", "short_conv", [](const std::string& prefix, const Json& p, const PartChildren&) {
+    return std::make_shared<ShortConv>(prefix, p);
+  });
+  register_part("mixer", "diff_attention", [](const std::string& prefix, const Json& p, const PartChildren& c) {
+    return std::make_shared<DiffAttention>(prefix, p, c);
+  });
+  register_part("ffn", "moe", [](const std::string& prefix, const Json& p, const PartChildren&) {
+    return std::make_shared<MoE>(prefix, p);
+  });
+  register_part("block", "post_norm",
+                [](const std::string& prefix, const Json&, const PartChildren& c) { return std::make_shared<PostNormBlock>(prefix, c); },
+                {{"norm1", "norm"}, {"mixer", "mixer"}, {"norm2", "norm?"}, {"ffn", "ffn?"}});
   register_part("embedding", "table", [](const std::string& prefix, const Json& p, const PartChildren& c) {
     return std::make_shared<Embedding>(prefix, p, c);
   });
@@ -1083,11 +1598,12 @@ void register_builtin_parts() {
     const int tied = (!t || t->is_null()) ? -1 : (t->as_bool() ? 1 : 0);
     return std::make_shared<LMHead>(prefix, param_int(p, "vocab"), param_int(p, "dim"), tied,
                                     p.has("tied_to") ? p.at("tied_to").as_string() : std::string(),
-                                    tensor_name(p, "tensor", prefix, "weight"));
+                                    tensor_name(p, "tensor", prefix, "weight"), p.has("scale") ? param_float(p, "scale") : 1.0);
   });
   register_part("norm", "rmsnorm", [](const std::string& prefix, const Json& p, const PartChildren&) {
     return std::make_shared<RMSNorm>(prefix, param_int(p, "dim"), param_float(p, "eps"), p.has("scalar") && p.at("scalar").as_bool(),
-                                     p.has("tensor") ? p.at("tensor").as_string() : std::string());
+                                     p.has("tensor") ? p.at("tensor").as_string() : std::string(),
+                                     p.has("one_plus") && p.at("one_plus").as_bool());
   });
   register_part("pos", "rope_neox", [](const std::string& prefix, const Json& p, const PartChildren&) {
     return std::make_shared<RotaryNeox>(prefix, param_int(p, "head_dim"), param_float(p, "theta"));
@@ -1295,6 +1811,36 @@ void RotaryNeox::upload(void* dst, const void* src, size_t bytes) {
 }
 void Sinusoidal::upload(void* dst, const void* src, size_t bytes) {
   if (hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice) != hipSuccess) throw KernelError("sinusoidal positions: copying the frequencies failed");
+}
+float DiffAttention::lambda_of(const Tensor l[4], int dk, double diff, bool on_host) {
+  std::vector<float> host((size_t)4 * dk);
+  for (int i = 0; i < 4; ++i) {
+    if (on_host) {
+      memcpy(host.data() + (size_t)i * dk, l[i].data, (size_t)dk * 4);
+    } else if (hipDeviceSynchronize() != hipSuccess ||
+               hipMemcpy(host.data() + (size_t)i * dk, l[i].data, (size_t)dk * 4, hipMemcpyDeviceToHost) != hipSuccess) {
+      throw KernelError("diff_attention: reading the lambda vectors back failed");
+    }
+  }
+  float s1 = 0.f, s2 = 0.f;
+  for (int d = 0; d < dk; ++d) {
+    s1 = std::fmaf(host[d], host[(size_t)dk + d], s1);
+    s2 = std::fmaf(host[(size_t)2 * dk + d], host[(size_t)3 * dk + d], s2);
+  }
+  return std::exp(s1) - std::exp(s2) + (float)diff;
+}
+void RMSNorm::plus_one(const Tensor& w, const Tensor& out, bool on_host) {
+  const size_t n = (size_t)w.numel();
+  if (on_host) {
+    for (size_t i = 0; i < n; ++i) out.ptr<float>()[i] = 1.0f + w.ptr<float>()[i];
+    return;
+  }
+  std::vector<float> host(n);
+  // the weight may still be on its way from the file: wait for every stream before reading it back
+  if (hipDeviceSynchronize() != hipSuccess || hipMemcpy(host.data(), w.data, n * 4, hipMemcpyDeviceToHost) != hipSuccess)
+    throw KernelError("rmsnorm: reading the weight back failed");
+  for (float& v : host) v = 1.0f + v;
+  if (hipMemcpy(out.data, host.data(), n * 4, hipMemcpyHostToDevice) != hipSuccess) throw KernelError("rmsnorm: writing the gain failed");
 }
 void RMSNorm::spread(const Tensor& one, const Tensor& all, bool on_host) {
   float g = 0.f;
