@@ -103,14 +103,15 @@ def diff_attention(h: np.ndarray, w: Dict[str, np.ndarray], prefix: str, m: dict
     q = h @ w[prefix + ".q"].T
     k = h @ w[prefix + ".k"].T
     v = h @ w[prefix + ".v"].T
-    q = short_conv(q, w[prefix + ".q.conv"]).reshape(T, H, 2, d)
-    k = short_conv(k, w[prefix + ".k.conv"]).reshape(T, G, 2, d)
-    v = short_conv(v, w[prefix + ".v.conv"]).reshape(T, G, dv)
+    if m.get("conv"):
+        q, k, v = (short_conv(u, w[f"{prefix}.{n}.conv"]) for u, n in ((q, "q"), (k, "k"), (v, "v")))
+    q, k, v = q.reshape(T, H, 2, d), k.reshape(T, G, 2, d), v.reshape(T, G, dv)
     q = rms_unit(q, eps) * w[prefix + ".q.norm"]
     k = rms_unit(k, eps) * w[prefix + ".k.norm"]
-    q = rotate_half_partial(q, range(T), m["rot"])
-    k = rotate_half_partial(k, range(T), m["rot"])
-    visible = block_mask(T, m["mask"]["size"])
+    if m.get("rot"):
+        q = rotate_half_partial(q, range(T), m["rot"])
+        k = rotate_half_partial(k, range(T), m["rot"])
+    visible = block_mask(T, m["mask"]["size"] if m.get("mask") else T)
     lam = differential_lambda(w, prefix, m["diff"])
     per = H // G
     out = np.zeros((T, H, dv))

@@ -80,7 +80,7 @@ Json mumasun_typed_config(const Json& d) {
     mo.set("kv_heads", kv);
     mo.set("dim", dim);
     mo.set("vdim", given(m, "vdim") ? need_int(m, "vdim", mw) : dim);
-    mo.set("conv", given(m, "conv") ? need_int(m, "conv", mw) : 1);
+    mo.set("conv", given(m, "conv") ? Json(need_int(m, "conv", mw)) : Json());      // one tap: a factor per channel
     mo.set("diff", need_float(m, "diff", mw));
     mo.set("scale", given(m, "scale") ? need_float(m, "scale", mw) : 1.0 / std::sqrt((double)dim));
     if (given(m, "mask")) {
@@ -186,7 +186,7 @@ ModelSpec mumasun_spec(const Json& config) {
       if (m.at("rot").has("scaling")) pos.params.set("scaling", m.at("rot").at("scaling"));
       mix.params.set("pos", pos.to_json());
     }
-    if (m.at("conv").as_int() > 1) {
+    if (m.has("conv")) {
       const std::string base = ls.prefix + ".mix.";
       PartSpec conv;
       conv.kind = "short_conv";

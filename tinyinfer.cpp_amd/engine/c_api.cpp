@@ -1258,6 +1258,34 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
   } else if (op == "gated_head_norm") {
     // o, proj, w, out; gate column, eps, heads, dv
     ops.gated_head_norm(arg(0), arg(1), (int)num(0), arg(2), (float)num(1), arg(3), (int)num(2), (int)num(3));
+  } else if (op == "norm_residual") {
+    // x, y, gain, gather [M, n] (may be absent); eps, accumulate
+    const bool g = n_t > 3 && arg(3).defined();
+    ops.norm_residual(arg(0), arg(1), arg(2), (float)num(0), num(1) != 0, g ? iptr(3) : nullptr, g ? (int)arg(3).shape[1] : 0);
+  } else if (op == "round_rows") {
+    ops.round_rows(arg(0), arg(1));
+  } else if (op == "scale") {
+    ops.scale(arg(0), (float)num(0));
+  } else if (op == "short_conv") {
+    // u, taps, state, entries [R, 4], entry of every row, positions, out
+    ops.short_conv(arg(0), arg(1), arg(2), iptr(3), (int)arg(3).shape[0], iptr(4), iptr(5), arg(6));
+  } else if (op == "diff_qk_prep") {
+    // qkv, q_w, k_w, inv_freq, rope_table, positions, slots, table, pool, q_out; eps, heads, kv_heads, dk, dv, rotated entries, mag
+    Ops::Rotation r = rotation(3, 4);
+    r.dims = (int)num(5);
+    r.mag = (float)num(6);
+    ops.diff_qk_prep(arg(0), fptr(1), fptr(2), (float)num(0), r, iptr(5), iptr(6), view_of(7, arg(8)), arg(8), arg(9), (int)num(1),
+                     (int)num(2), (int)num(3), (int)num(4));
+  } else if (op == "diff_attention") {
+    // q, pool, table, positions, slots, out; heads, kv_heads, dk, dv, scale, block, window, lambda, eps, out_scale
+    ops.diff_attention(arg(0), arg(1), view_of(2, arg(1)), iptr(3), iptr(4), arg(5), (int)num(0), (int)num(1), (int)num(2), (int)num(3),
+                       (float)num(4), (int)num(5), (int)num(6), (float)num(7), (float)num(8), (float)num(9));
+  } else if (op == "moe_route") {
+    // h, router, ids, wts; top, score kind, renormalize
+    ops.moe_route(arg(0), arg(1), arg(2), arg(3), (int)num(0), (Ops::RouterScore)(int)num(1), num(2) != 0);
+  } else if (op == "moe_experts") {
+    // h, ids, wts, up, down, y; experts, scale_input
+    ops.moe_experts(arg(0), arg(1), arg(2), arg(3), arg(4), arg(5), (int)num(0), num(1) != 0);
   } else if (op == "argmax") {
     ops.argmax(arg(0), arg(1).ptr<int>());
   } else if (op == "sample") {

@@ -96,7 +96,9 @@ _LIB_OF = {"embed": "core", "rmsnorm": "core", "rope_neox": "core", "rope_table"
            "qk_norm_inplace": "core", "argmax": "sampling", "sample": "sampling", "attention_rows": "attention_generic",
            "fill_random": "core", "fill_zero": "core", "add_sinusoid": "pointwise", "add_row": "pointwise", "xielu": "pointwise",
            "scaled_add": "pointwise", "qkv_split_write": "pointwise", "attention_capped": "attention_generic",
-           "mlstm_scan": "recurrent", "gated_head_norm": "recurrent"}
+           "mlstm_scan": "recurrent", "gated_head_norm": "recurrent", "norm_residual": "residual", "round_rows": "residual",
+           "scale": "residual", "short_conv": "diff_attention", "diff_qk_prep": "diff_attention", "diff_attention": "diff_attention",
+           "moe_route": "moe", "moe_experts": "moe"}
 
 
 class Ops:
@@ -351,6 +353,39 @@ class Ops:
 
     def gated_head_norm(self, o, proj, gate_col, w, eps, out, heads, dv):
         self._call("gated_head_norm", [o, proj, w, out], [gate_col, eps, heads, dv])
+
+    # ---- post-norm layers, short convolutions, differential attention, mixtures of experts
+    def norm_residual(self, x, y, gain, eps, accumulate=True, gather=None):
+        """x (+)= y / rms(y) * gain, all float32; gather int32 [M, n]: row m of y is the sum of the rows y[gather[m, k]]."""
+        self._call("norm_residual", [x, y, gain, gather], [eps, int(bool(accumulate))])
+
+    def round_rows(self, x, out):
+        self._call("round_rows", [x, out])
+
+    def scale(self, x, s):
+        self._call("scale", [x], [s])
+
+    def short_conv(self, u, taps, state, entries, entry_of, positions, out):
+        """out[m, c] = sum_j taps[c, j] u(pos[m] - (K - 1) + j)[c]; state f32 [slots, K - 1, C] holds the rows before each
+        entry's start and is left with the last K - 1 rows; entries int32 [R, 4] = (first row, tokens, start, slot)."""
+        self._call("short_conv", [u, taps, state, entries, entry_of, positions, out])
+
+    def diff_qk_prep(self, qkv, q_w, k_w, inv_freq, rope_table, positions, slots, table, pool, q_out, eps, heads, kv_heads, dk, dv,
+                     rot_dims=0, mag=1.0):
+        """qkv f32 [M, heads 2 dk + kv_heads (2 dk + dv)]; pool [pages, kv_heads, P, 2 dk + dv] (K [kv][P][2 dk] | V [kv][dv][P])."""
+        self._call("diff_qk_prep", [qkv, q_w, k_w, inv_freq, rope_table, positions, slots, table, pool, q_out],
+                   [eps, heads, kv_heads, dk, dv, rot_dims, mag])
+
+    def diff_attention(self, q, pool, table, positions, slots, out, heads, kv_heads, dk, dv, scale, lam, eps, out_scale, block=0, window=0):
+        self._call("diff_attention", [q, pool, table, positions, slots, out],
+                   [heads, kv_heads, dk, dv, scale, int(block or 0), int(window or 0), lam, eps, out_scale])
+
+    def moe_route(self, h, router, ids, wts, top, score="sigmoid", renormalize=False):
+        self._call("moe_route", [h, router, ids, wts], [top, {"sigmoid": 0, "softmax": 1}[score], int(bool(renormalize))])
+
+    def moe_experts(self, h, ids, wts, up, down, y, experts, scale_input=True):
+        """y f32 [M, W] = sum over a token's experts; up [experts F, W], down [experts W, F]."""
+        self._call("moe_experts", [h, ids, wts, up, down, y], [experts, int(bool(scale_input))])
 
     def argmax(self, logits, out):
         if out.dtype != native.torch().int32 or out.shape[0] < logits.shape[0]:

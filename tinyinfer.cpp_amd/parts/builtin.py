@@ -174,8 +174,12 @@ class NativeBlock(NativePart):
         self._call("forward", native_context(ctx, x.shape[0]), [x])
 
 
+class NativeFilter(NativePart):
+    """An operation along time on the channels of a step's rows (it runs inside the part that owns it)."""
+
+
 FAMILY_VIEWS = {"embedding": NativeEmbedding, "head": NativeHead, "norm": NativeNorm, "pos": NativePos, "mixer": NativeMixer,
-                "ffn": NativeMixer, "block": NativeBlock}
+                "ffn": NativeMixer, "block": NativeBlock, "filter": NativeFilter}
 
 
 # ------------------------------------------------------- the built-in kinds, by name

@@ -1796,6 +1796,7 @@ std::shared_ptr<Part> make_foreign_part(const std::string& family, uint64_t id, 
   if (family == "ffn") return std::make_shared<ForeignFFN>(id, prefix, description, children);
   if (family == "block") return std::make_shared<ForeignBlock>(id, prefix, description, children);
   if (family == "head") return std::make_shared<ForeignHead>(id, prefix, description, children);
+  if (family == "filter") throw ConfigError("a filter part is implemented in the library or in a plugin loaded into it, not through the call table");
   throw ConfigError("unknown part family '" + family + "'");
 }
 

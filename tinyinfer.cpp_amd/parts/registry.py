@@ -1,6 +1,6 @@
 """Registry of parts by family and kind.
 
-Families: "embedding", "norm", "pos", "mixer", "ffn", "block", "head".
+Families: "embedding", "norm", "pos", "mixer", "ffn", "block", "head", "filter".
 There is one table, the host library's (parts/parts.cpp `register_part`).  A kind
 registered from Python is entered there too, with a factory that calls back into
 the Python class, so a `ModelSpec` that names it is built by the library like any
@@ -15,7 +15,7 @@ from typing import Callable, Dict, Tuple
 
 from .. import native
 
-FAMILIES = ("embedding", "norm", "pos", "mixer", "ffn", "block", "head")
+FAMILIES = ("embedding", "norm", "pos", "mixer", "ffn", "block", "head", "filter")
 _PARTS: Dict[Tuple[str, str], Callable] = {}
 
 

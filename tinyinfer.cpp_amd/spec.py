@@ -122,11 +122,14 @@ class PagedKVNeed:
     head_dim: int
     window: Optional[int] = None
     v_dim: Optional[int] = None      # the size of a value where it differs from head_dim
+    block: Optional[int] = None      # tokens read only positions of their own block of this many: pages before it go back
 
     def to_dict(self) -> dict:
         d = {"kind": "paged_kv", "kv_heads": self.kv_heads, "head_dim": self.head_dim, "window": self.window}
         if self.v_dim:
             d["v_dim"] = self.v_dim
+        if self.block:
+            d["block"] = self.block
         return d
 
 
@@ -159,4 +162,4 @@ def cache_need_from_dict(d):
         return StateNeed(tuple(d["shape"]))
     if d["kind"] == "paged_rows":
         return PagedRowsNeed(tuple(d["row_shape"]), bool(d.get("float32")), d.get("window"))
-    return PagedKVNeed(d["kv_heads"], d["head_dim"], d.get("window"), d.get("v_dim"))
+    return PagedKVNeed(d["kv_heads"], d["head_dim"], d.get("window"), d.get("v_dim"), d.get("block"))
