@@ -139,7 +139,8 @@ def plain_maps(q, k, v, scale, block, lam, eps, out_scale, per):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("heads,kv,dk,dv,P,block,rot_dims", [(4, 2, 16, 24, 16, 40, 8), (3, 3, 7, 9, 4, 13, 6), (6, 1, 40, 33, 64, 150, 40),
                                                               (2, 2, 32, 64, 16, 64, 32), (2, 1, 64, 32, 16, 100, 0), (1, 1, 130, 256, 8, 50, 2),
-                                                              (2, 1, 24, 16, 16, 1000, 12)])
+                                                              (2, 1, 24, 16, 16, 1000, 12), (16, 2, 128, 128, 32, 40, 64), (4, 4, 64, 128, 16, 70, 20),
+                                                              (3, 1, 32, 32, 16, 33, 32)])
 def test_prepared_keys_and_differential_attention(ops, dtype, heads, kv, dk, dv, P, block, rot_dims):
     """q/k/v of a whole request normed, rotated and written in two portions, then the attention of every row.  On the
     entries that are not rotated, the last row's first map points at the second key of its block (far back), and its
@@ -201,6 +202,23 @@ def test_prepared_keys_and_differential_attention(ops, dtype, heads, kv, dk, dv,
     err = np.abs(f64(out) - want)
     bound = 2e-4 if dtype == "float32" else 3e-2           # the output is normed: entries of order one
     assert err.max() < bound, (np.unravel_index(err.argmax(), err.shape), err.max())
+    if dtype == "bfloat16" and dk in (32, 64, 128) and dv in (32, 64, 128) and P % 16 == 0:
+        # the matrix-core kernels: the request as one portion in tiles of 64 rows (the last one short), then every row as a
+        # single token (a step of decoded tokens), then some rows as tiles beside others as single tokens
+        entries = dev([[0, T, 0, 0]], torch.int32)
+        tiles = dev([[0, r, min(64, T - r)] for r in range(0, T, 64)], torch.int32)
+        args = (q_out, pool, dev(table, torch.int32), dev(pos, torch.int32), dev(slots, torch.int32))
+        calls = ops.timing_report() and None
+        ops.count_calls(True)
+        for lists in (dict(tiles=tiles, entries=entries), dict(all_rows=True),
+                      dict(tiles=tiles[:1], entries=entries, rows=dev(list(range(64, T)), torch.int32))):
+            fast = torch.zeros(T, heads * dv, device="cuda", dtype=DT[dtype])
+            ops.diff_attention(*args, fast, heads, kv, dk, dv, scale, lam, eps, out_scale, block=block, **lists)
+            err = np.abs(f64(fast) - want)
+            assert err.max() < bound, (list(lists), np.unravel_index(err.argmax(), err.shape), err.max())
+        took = [c["name"] for c in ops.timing_report()]
+        ops.count_calls(False)
+        assert took and all("[mfma]" in n for n in took), took
     # no blocks: every earlier key is visible
     ops.diff_attention(q_out, pool, dev(table, torch.int32), dev(pos, torch.int32), dev(slots, torch.int32), out, heads, kv, dk, dv, scale,
                        lam, eps, out_scale, block=0)

@@ -36,6 +36,7 @@ HEADERS = ["common.h", "qk_prep.h", "tinyinfer_kernels.h", "tinyinfer_kernels_tu
 # on every turn of the loop, so their MFMAs are told to work on ordinary vector registers.
 EXTRA_FLAGS: Dict[str, List[str]] = {
     "attention_bf16": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "diff_attention_bf16": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
 }
 
 def _discover() -> Dict[str, str]:
@@ -51,7 +52,7 @@ ON_DEMAND = ("measure",)
 
 # libraries that only some architectures call into (by the name config.json gives the architecture); every other
 # library serves them all
-ONLY_FOR = {"pointwise": ("Miterax",), "recurrent": ("Miterax",), "residual": ("Mumasun",), "diff_attention": ("Mumasun",),
+ONLY_FOR = {"pointwise": ("Miterax",), "recurrent": ("Miterax",), "residual": ("Mumasun",), "diff_attention": ("Mumasun",), "diff_attention_bf16": ("Mumasun",),
             "moe": ("Mumasun",)}
 # ... and libraries that a named architecture never calls into
 NOT_FOR = {"attention_generic": ("Mumasun",), "attention_bf16": ("Mumasun",)}

@@ -162,6 +162,19 @@ int ti_diff_attention_rows(int dtype, const void* q, const void* pool, const int
                            const int* slot, void* out, int M, int n_head, int n_kv, int dk, int dv, int page_size, float scale,
                            int block, int window, float lambda, float eps, float out_scale, hipStream_t stream);
 
+// ---- libti_diff_attention_bf16: the same attention on the matrix cores (dk, dv in {32, 64, 128}, pages of 16 n rows);
+// 3: sizes not served.  tiles int32 [n_tiles][3] = (entry, first row, rows <= 64) of entries int32 [.][4] = (row0, tokens,
+// start, -); the block table's row of an entry is the entry's index
+int ti_diff_attention_tiles_bf16(const void* q, const void* pool, const int* table, int table_stride, const int* tiles,
+                                 const int* entries, void* out, int n_tiles, int n_head, int n_kv, int dk, int dv,
+                                 int page_size, float scale, int block, int window, float lambda, float eps, float out_scale,
+                                 hipStream_t stream);
+// single rows (rows int32 [n_rows], or null: rows 0 .. n_rows - 1); at most 16 query heads a kv head
+int ti_diff_attention_rows_bf16(const void* q, const void* pool, const int* table, int table_stride, const int* pos,
+                                const int* slot, const int* rows, void* out, int n_rows, int n_head, int n_kv, int dk, int dv,
+                                int page_size, float scale, int block, int window, float lambda, float eps, float out_scale,
+                                hipStream_t stream);
+
 // ---- libti_moe: a mixture of experts
 // scores (score_kind 0: sigmoid, 1: softmax over the experts) of h [M, W] against router f32 [E, W] in 32-bit; the `top`
 // largest per token (ties: the lower index) to ids int32 [M, top] and wts f32 [M, top] (renormalize: divided by their sum)

@@ -1277,9 +1277,23 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
     ops.diff_qk_prep(arg(0), fptr(1), fptr(2), (float)num(0), r, iptr(5), iptr(6), view_of(7, arg(8)), arg(8), arg(9), (int)num(1),
                      (int)num(2), (int)num(3), (int)num(4));
   } else if (op == "diff_attention") {
-    // q, pool, table, positions, slots, out; heads, kv_heads, dk, dv, scale, block, window, lambda, eps, out_scale
+    // q, pool, table, positions, slots, out, [tiles [n, 3], rows [n], entries [R, 4]]; heads, kv_heads, dk, dv, scale, block,
+    // window, lambda, eps, out_scale, [rows of single tokens where no list names them]
+    Ops::DiffAttentionLists l;
+    const bool listed = n_t > 8 || n_s > 10;
+    if (n_t > 6 && arg(6).defined()) {
+      l.tiles = iptr(6);
+      l.n_tiles = (int)arg(6).shape[0];
+    }
+    if (n_t > 7 && arg(7).defined()) {
+      l.rows = iptr(7);
+      l.n_rows = (int)arg(7).shape[0];
+    } else if (n_s > 10) {
+      l.n_rows = (int)num(10);
+    }
+    if (n_t > 8) l.entry_meta = iptr(8);
     ops.diff_attention(arg(0), arg(1), view_of(2, arg(1)), iptr(3), iptr(4), arg(5), (int)num(0), (int)num(1), (int)num(2), (int)num(3),
-                       (float)num(4), (int)num(5), (int)num(6), (float)num(7), (float)num(8), (float)num(9));
+                       (float)num(4), (int)num(5), (int)num(6), (float)num(7), (float)num(8), (float)num(9), listed ? &l : nullptr);
   } else if (op == "moe_route") {
     // h, router, ids, wts; top, score kind, renormalize
     ops.moe_route(arg(0), arg(1), arg(2), arg(3), (int)num(0), (Ops::RouterScore)(int)num(1), num(2) != 0);

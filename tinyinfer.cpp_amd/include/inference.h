@@ -366,9 +366,14 @@ class Ops {
                     int dk, int dv);
   // differential attention of every row over such pages: (a1 - lambda a2) / rms * out_scale per head; a key is visible
   // inside the query's block of `block` positions (0: no blocks) and window (0: none)
+  // lists (device int32, the step's metadata): tiles [n_tiles][3] = (entry, first row, rows <= 64) of the entries of several
+  // tokens, rows [n_rows] the rows of single-token entries (null with n_rows = M: every row is one).  With them the bfloat16
+  // matrix-core kernels serve the sizes they take; without, or for other sizes and float32, every row is walked on its own
+  struct DiffAttentionLists { const int* tiles = nullptr; int n_tiles = 0; const int* rows = nullptr; int n_rows = 0;
+                              const int* entry_meta = nullptr; };
   void diff_attention(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
                       const Tensor& out, int heads, int kv_heads, int dk, int dv, float scale, int block, int window, float lambda,
-                      float eps, float out_scale);
+                      float eps, float out_scale, const DiffAttentionLists* lists = nullptr);
   enum RouterScore { Sigmoid = 0, Softmax = 1 };
   // the `top` experts with the largest scores of h against router f32 [E, W]: ids int32 [M, top], wts f32 [M, top]
   void moe_route(const Tensor& h, const Tensor& router, const Tensor& ids, const Tensor& wts, int top, RouterScore score,

@@ -376,9 +376,20 @@ class Ops:
         self._call("diff_qk_prep", [qkv, q_w, k_w, inv_freq, rope_table, positions, slots, table, pool, q_out],
                    [eps, heads, kv_heads, dk, dv, rot_dims, mag])
 
-    def diff_attention(self, q, pool, table, positions, slots, out, heads, kv_heads, dk, dv, scale, lam, eps, out_scale, block=0, window=0):
-        self._call("diff_attention", [q, pool, table, positions, slots, out],
-                   [heads, kv_heads, dk, dv, scale, int(block or 0), int(window or 0), lam, eps, out_scale])
+    def diff_attention(self, q, pool, table, positions, slots, out, heads, kv_heads, dk, dv, scale, lam, eps, out_scale, block=0, window=0,
+                       tiles=None, rows=None, entries=None, all_rows=False):
+        """tiles int32 [n, 3] = (entry, first row, rows <= 64) with entries int32 [R, 4] = (row0, tokens, start, -), rows int32 [n]
+        (or all_rows: every row is a single token): the lists of the bfloat16 matrix-core kernels; without them every row is
+        walked on its own."""
+        tensors, numbers = [q, pool, table, positions, slots, out], [heads, kv_heads, dk, dv, scale, int(block or 0), int(window or 0), lam, eps, out_scale]
+        libs = ["diff_attention"]
+        if tiles is not None or rows is not None or all_rows:
+            tensors += [tiles, rows, entries]
+            if all_rows:
+                numbers.append(q.shape[0])
+            if q.dtype == native.torch().bfloat16:
+                libs.append("diff_attention_bf16")
+        self._call("diff_attention", tensors, numbers, libs=libs)
 
     def moe_route(self, h, router, ids, wts, top, score="sigmoid", renormalize=False):
         self._call("moe_route", [h, router, ids, wts], [top, {"sigmoid": 0, "softmax": 1}[score], int(bool(renormalize))])

@@ -1063,13 +1063,33 @@ void Ops::diff_qk_prep(const Tensor& qkv, const float* q_w, const float* k_w, fl
 
 void Ops::diff_attention(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
                          const Tensor& out, int heads, int kv_heads, int dk, int dv, float scale, int block, int window, float lambda,
-                         float eps, float out_scale) {
+                         float eps, float out_scale, const DiffAttentionLists* lists) {
   TIMED("diff_attention " + dims(q));
   const int64_t M = q.shape[0];
   require(q.ndim == 2 && q.shape[1] == (int64_t)heads * 2 * dk && out.ndim == 2 && out.shape[0] == M &&
               out.shape[1] == (int64_t)heads * dv && q.dtype == pool.dtype && out.dtype == q.dtype && q.contiguous() && out.contiguous(),
           "diff_attention: q/out/pool shapes or dtypes do not fit");
   check_split_pool("diff_attention", pool, kv_heads, 2 * dk, dv, q.dtype);
+  if (M == 0) return;
+  if (lists && q.dtype == DType::BF16 && use.fast_attention && kernel_library_available("diff_attention_bf16") &&
+      (lists->n_tiles == 0 || (lists->tiles && lists->entry_meta))) {
+    int rc = 0;
+    if (lists->n_tiles)
+      rc = KERNEL("diff_attention_bf16", ti_diff_attention_tiles_bf16)(q.data, pool.data, view.table, view.table_width, lists->tiles,
+                                                                       lists->entry_meta, out.data, lists->n_tiles, heads, kv_heads, dk,
+                                                                       dv, (int)pool.shape[2], scale, block, window, lambda, eps,
+                                                                       out_scale, (hipStream_t)launch_stream());
+    if (rc == 0 && lists->n_rows)
+      rc = KERNEL("diff_attention_bf16", ti_diff_attention_rows_bf16)(q.data, pool.data, view.table, view.table_width, positions, slots,
+                                                                      lists->rows, out.data, lists->n_rows, heads, kv_heads, dk, dv,
+                                                                      (int)pool.shape[2], scale, block, window, lambda, eps, out_scale,
+                                                                      (hipStream_t)launch_stream());
+    if (rc == 0) {
+      took("[mfma]");
+      return;
+    }
+    if (rc != 3) check("diff_attention_bf16", rc, "diff_attention(bf16)");     // 3: sizes not served: every row on its own below
+  }
   took("[generic]");
   int rc = KERNEL("diff_attention", ti_diff_attention_rows)(code(q.dtype, "diff_attention"), q.data, pool.data, view.table,
                                                             view.table_width, positions, slots, out.data, (int)M, heads, kv_heads, dk,

@@ -1392,6 +1392,46 @@ class DiffAttention final : public MixerPart {
     n.block = block;
     return n;
   }
+  // The lists of the matrix-core kernels: tiles of TILE_ROWS query rows over the entries of several tokens, and the rows
+  // of single-token entries.  Every such mixer of a model asks for the same lists; the first one builds them.
+  static constexpr int TILE_ROWS = 64;
+  void plan(StepPlan& plan) const override {
+    if (plan.decode_only() || plan.has("dattn.tiles")) return;
+    const auto& entries = plan.entries();
+    size_t n_tiles = 0, n_rows = 0;
+    for (const auto& e : entries) {
+      if (e.n_tokens > 1) n_tiles += (size_t)(e.n_tokens + TILE_ROWS - 1) / TILE_ROWS;
+      else ++n_rows;
+    }
+    int* tiles = plan.ints("dattn.tiles", 3 * n_tiles);
+    int* rows = plan.ints("dattn.rows", n_rows);
+    size_t t = 0, r = 0;
+    for (size_t i = 0; i < entries.size(); ++i) {
+      const auto& e = entries[i];
+      if (e.n_tokens == 1) {
+        rows[r++] = e.row0;
+        continue;
+      }
+      for (int q0 = 0; q0 < e.n_tokens; q0 += TILE_ROWS) {
+        tiles[t++] = (int)i;
+        tiles[t++] = e.row0 + q0;
+        tiles[t++] = std::min(TILE_ROWS, e.n_tokens - q0);
+      }
+    }
+  }
+  Ops::DiffAttentionLists lists(const StepContext& ctx) const {
+    Ops::DiffAttentionLists l;
+    l.entry_meta = ctx.entry_meta;
+    if (ctx.decode_only) {
+      l.n_rows = (int)ctx.M;
+      return l;
+    }
+    l.tiles = ctx.planned("dattn.tiles");
+    l.n_tiles = (int)(ctx.planned_size("dattn.tiles") / 3);
+    l.rows = ctx.planned("dattn.rows");
+    l.n_rows = (int)ctx.planned_size("dattn.rows");
+    return l;
+  }
   void run(StepContext& ctx, const Rows& h, const Tensor& out, Ops::Epilogue epi) {
     const int64_t M = h.t.shape[0];
     const int64_t width = nq + nk + nv;
@@ -1411,8 +1451,9 @@ class DiffAttention final : public MixerPart {
     ctx.ops.diff_qk_prep(qkv, q_norm_w.ptr<float>(), k_norm_w.ptr<float>(), eps, rot, ctx.positions, ctx.slots, view, pool, q, heads,
                          kv_heads, dk, dv);
     Tensor a = ctx.buf("dattn.out", ctx.act_dtype, {M, no});
+    const Ops::DiffAttentionLists l = lists(ctx);
     ctx.ops.diff_attention(q, pool, view, ctx.positions, ctx.slots, a, heads, kv_heads, dk, dv, scale, block, window, lambda, eps,
-                           (float)(1.0 - diff));
+                           (float)(1.0 - diff), ctx.plan ? &l : nullptr);
     ctx.ops.linear(a, w_o, out, epi, false);
   }
   void forward(StepContext& ctx, const Rows& h, const Tensor& x) override { run(ctx, h, x, Ops::Add); }
