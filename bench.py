@@ -27,6 +27,13 @@ every layer), `mlstm` (an mLSTM in every layer, as many heads as the model has k
 heads) or `alternate` (attention, mLSTM, attention, ...).  Run it beside the default
 design with the same `--model` and `--layers`; the default workload and its line stay
 as they are.
+
+`--design mumasun` does the same for a Mumasun decoder: post-norm layers, differential
+attention with as many query and kv heads as the model has, two maps of half the head
+size each over values of the full head size (the projections have the sizes of the
+model's own), a short convolution of four taps, keys visible inside blocks of
+`--mask-size` positions, and `--experts` experts of which a token takes `--top`, each
+sized so that a token's experts do the arithmetic of the model's dense feed-forward.
 """
 from __future__ import annotations
 
@@ -71,6 +78,19 @@ def miterax_config(base, mixers):
                 layers=[kinds[i % len(kinds)] for i in range(L)])
 
 
+def mumasun_config(base, experts, top, mask_size):
+    """A Mumasun config.json with the layer widths of the Qwen3 configuration `base`."""
+    H, F, hd = base["hidden_size"], base["intermediate_size"], base["head_dim"]
+    ff = max(64, (3 * F // (2 * top)) // 64 * 64)        # top experts of two matrices do what three dense ones of F do
+    layer = dict(type="attention",
+                 mixer=dict(heads=base["num_attention_heads"], kv_heads=base["num_key_value_heads"], dim=hd // 2, vdim=hd, conv=4,
+                            diff=0.5, scale=(hd // 2) ** -0.5, mask=dict(size=mask_size),
+                            rot=dict(base=1000000.0, dims=hd // 2, scaling=dict(factor=4.0, original=8192, fast=32.0, slow=1.0))),
+                 mlp=dict(kind="moe", expert=dict(ff=ff), router=dict(experts=experts, top=top)))
+    return dict(architecture="Mumasun", width=H, vocab=base["vocab_size"], logit_scale=1.0, norm=dict(eps=1e-6),
+                layers=[layer] * base["num_hidden_layers"])
+
+
 MAX_SEQ = 4096            # context length a request may reach (more if --context asks for it)
 PAGE = 16
 PEAK_HBM = 8.0e12         # bytes/s, MI355X
@@ -88,9 +108,11 @@ def model_numbers(model):
     per token; per cached token it reads the keys and values of every cache layer."""
     seen = set()
     layer_params = head_params = vector_params = embed_row = 0
-    attn = []                     # (heads, head_dim, window) of every mixer that attends over cached keys
+    routed = []                   # (parameters of all experts, experts, top) of every routed feed-forward
+    attn = []                     # (heads, summed size of the score products, of the value products, window, block) per attending mixer
     cells = []                    # shape of the per-request state of every recurrent mixer
     for part in model.parts():
+        experts = 0
         for name, need in part.tensors().items():
             n = 1
             for d in need.shape:
@@ -105,22 +127,32 @@ def model_numbers(model):
                 vector_params += n
             elif part.family == "head":
                 head_params += n
+            elif part.family == "ffn" and getattr(part, "kind", "") == "moe":
+                experts += n                          # a token reads `top` of them, a step those its tokens chose
             else:
                 layer_params += n
+        if experts:
+            routed.append((experts, part.params["experts"], part.params["top"]))
         need = part.cache_need()
         if need is not None and hasattr(need, "kv_heads") and "heads" in getattr(part, "params", {}):
-            attn.append((part.params["heads"], need.head_dim, need.window))
+            v = getattr(need, "v_dim", None) or need.head_dim
+            two_maps = getattr(part, "kind", "") == "diff_attention"     # its keys hold two maps; both read the values
+            attn.append((part.params["heads"], need.head_dim, 2 * v if two_maps else v, need.window, getattr(need, "block", None)))
         if need is not None and hasattr(need, "shape") and not hasattr(need, "kv_heads"):
             cells.append(tuple(need.shape))
-    weight_bytes = (layer_params + head_params) * 2 + vector_params * 4 + embed_row * 2
+    # what a token's experts hold, and what a step of `batch` tokens reads of the experts if every token chooses alike at random
+    active = sum(n * top / e for n, e, top in routed)
+    expert_read = lambda batch: sum(n * (1.0 - (1.0 - top / e) ** batch) for n, e, top in routed)      # noqa: E731
+    weight_bytes_at = lambda batch: (layer_params + head_params + expert_read(batch)) * 2 + vector_params * 4 + embed_row * 2      # noqa: E731
+    weight_bytes = weight_bytes_at(1 << 20)
     # per cached token the keys and values of every cache layer (values of their own size where they have one); per
     # request the 32-bit state of every recurrent layer, read and written once a step
     state_bytes = sum(2 * 4 * int(np_prod(need.shape)) * n for need, n in model.cache_groups if not hasattr(need, "kv_heads") and hasattr(need, "shape"))
     kv_bytes = lambda context: state_bytes + sum(need.kv_heads * (need.head_dim + (getattr(need, "v_dim", None) or need.head_dim)) * 2 * n *      # noqa: E731
-                                                 min(context, need.window or context)
+                                                 min(context, need.window or context, getattr(need, "block", None) or context)
                                                  for need, n in model.cache_groups if hasattr(need, "kv_heads"))
-    return dict(layer_params=layer_params, head_params=head_params, weight_bytes=weight_bytes, kv_bytes=kv_bytes, attention=attn,
-                cells=cells, state_bytes=state_bytes)
+    return dict(layer_params=layer_params + active, head_params=head_params, weight_bytes=weight_bytes, weight_bytes_at=weight_bytes_at,
+                kv_bytes=kv_bytes, attention=attn, cells=cells, state_bytes=state_bytes, routed=routed)
 
 
 def np_prod(shape):
@@ -133,7 +165,12 @@ def np_prod(shape):
 def prefill_flops(model, T):
     n = model_numbers(model)
     gemm = 2.0 * n["layer_params"] * T + 2.0 * n["head_params"]              # the head runs on one row
-    attn = sum(2.0 * hd * T * (T + 1) * heads for heads, hd, _ in n["attention"])   # QK^T and PV over the causal half
+    def visible(window, block):       # pairs (query, key) that count: the causal half, cut by a block's start or a window
+        if block:
+            full, rest = divmod(T, block)
+            return full * block * (block + 1) / 2.0 + rest * (rest + 1) / 2.0
+        return T * (T + 1) / 2.0
+    attn = sum(2.0 * (qk + pv) * visible(w, b) * heads for heads, qk, pv, w, b in n["attention"])   # QK^T and PV over the visible pairs
     cells = sum(6.0 * np_prod(shape) * T for shape in n["cells"])                   # decay, outer product and read-out of a memory
     return gemm + attn + cells
 
@@ -190,7 +227,10 @@ def decode_floor(engine, rids, last, nums, context, batch):
     sizes = []
     for c in calls:
         m = re.search(r"\* (\d+)x(\d+)", c["name"])
-        per_call = int(m.group(1)) * int(m.group(2)) * 2 if m else kv_layer if c["name"].startswith("attention") else 4096
+        per_call = int(m.group(1)) * int(m.group(2)) * 2 if m else kv_layer if c["name"].startswith(("attention", "diff_attention")) else 4096
+        if c["name"].startswith("moe_experts") and nums["routed"]:
+            n_all, e, top = nums["routed"][0]
+            per_call = int(n_all * (1.0 - (1.0 - top / e) ** batch) * 2)      # the experts the step's tokens chose
         if c["name"].startswith("mlstm_scan") and nums["cells"]:
             per_call = 2 * 4 * np_prod(nums["cells"][0]) * batch      # the requests' state, read and written
         sizes += [per_call] * c["calls"]
@@ -366,8 +406,11 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--model", choices=sorted(MODELS), default="0.6b", help="whose layer sizes the model has")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
-    ap.add_argument("--design", choices=["qwen3", "miterax"], default="qwen3",
-                    help="miterax: a Miterax decoder with the layer widths of --model instead (see --mixers)")
+    ap.add_argument("--design", choices=["qwen3", "miterax", "mumasun"], default="qwen3",
+                    help="miterax / mumasun: a decoder of that design with the layer widths of --model instead (see --mixers; --experts, --top, --mask-size)")
+    ap.add_argument("--experts", type=int, default=8, help="--design mumasun: experts per layer")
+    ap.add_argument("--top", type=int, default=2, help="--design mumasun: experts a token takes")
+    ap.add_argument("--mask-size", type=int, default=4096, help="--design mumasun: positions of a block of visible keys")
     ap.add_argument("--mixers", choices=["attention", "mlstm", "alternate"], default="alternate",
                     help="--design miterax: the mixer of its layers")
     ap.add_argument("--batch", type=int, default=8)
@@ -403,6 +446,9 @@ def main() -> int:
     if args.design == "miterax":
         cfg = miterax_config(cfg, args.mixers)
         model_name = f"Miterax ({args.mixers} mixers) at {NAMES[args.model]} sizes"
+    if args.design == "mumasun":
+        cfg = mumasun_config(cfg, args.experts, args.top, args.mask_size)
+        model_name = f"Mumasun ({args.top} of {args.experts} experts, blocks of {args.mask_size}) at {NAMES[args.model]} sizes"
     rng = np.random.default_rng(0)
     context, prefill_tokens = args.context, args.prefill_tokens
     max_seq = max(MAX_SEQ, context + args.warmup + args.steps + 64, prefill_tokens, args.cached + args.portion)
@@ -454,7 +500,7 @@ def main() -> int:
                                                           f"p{b}_", draw=draw)[0], 1)
 
     ctx_mean = context + args.warmup + args.steps / 2.0
-    step_bytes = nums["weight_bytes"] + args.batch * nums["kv_bytes"](ctx_mean)
+    step_bytes = nums["weight_bytes_at"](args.batch) + args.batch * nums["kv_bytes"](ctx_mean)
     achieved = step_bytes / (ms * 1e-3) if ms else None
     roofline = prefill = None
     if achieved is not None:

@@ -229,7 +229,9 @@ def test_prepared_keys_and_differential_attention(ops, dtype, heads, kv, dk, dv,
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_router_and_experts(ops, dtype):
     rng = np.random.default_rng(11)
-    for M, W, E, top, F in [(9, 48, 5, 2, 40), (3, 50, 1, 1, 9), (17, 130, 70, 8, 33), (4, 64, 8, 8, 64)]:
+    # the last two: enough pairs for the grouped matrix-core path in bfloat16 (experts with no token, with one, with hundreds)
+    for M, W, E, top, F in [(9, 48, 5, 2, 40), (3, 50, 1, 1, 9), (17, 130, 70, 8, 33), (4, 64, 8, 8, 64), (300, 96, 11, 3, 160),
+                            (200, 64, 40, 1, 32)]:
         h = bf16_round(rng.normal(size=(M, W)))
         router = rng.normal(size=(E, W)) * 2 / math.sqrt(W)
         up = bf16_round(rng.normal(size=(E, F, W)) / math.sqrt(W))

@@ -53,7 +53,7 @@ ON_DEMAND = ("measure",)
 # libraries that only some architectures call into (by the name config.json gives the architecture); every other
 # library serves them all
 ONLY_FOR = {"pointwise": ("Miterax",), "recurrent": ("Miterax",), "residual": ("Mumasun",), "diff_attention": ("Mumasun",), "diff_attention_bf16": ("Mumasun",),
-            "moe": ("Mumasun",)}
+            "moe": ("Mumasun",), "moe_bf16": ("Mumasun",)}
 # ... and libraries that a named architecture never calls into
 NOT_FOR = {"attention_generic": ("Mumasun",), "attention_bf16": ("Mumasun",)}
 

@@ -1,0 +1,195 @@
+// The experts of a mixture of experts for steps of many tokens, bfloat16 on the matrix cores of gfx950.
+//
+//   1. moe_group: counts the (token, expert) pairs of every expert, lays the experts' runs of rows one after
+//      the other and cuts them into tiles of 64 rows: offsets, the list of tiles, cursors at zero.
+//   2. moe_place: every pair takes the next free row of its expert's run (which row does not matter: a row of
+//      a product depends on no other row) and writes its scaled input there, rounded to bfloat16.
+//   3. two grouped products over the tiles: act = relu(A up_e^T)^2 (bfloat16), out = act down_e^T (32-bit).
+//      Weights are the A operand of v_mfma_f32_16x16x32_bf16 and tokens the 16 columns, both straight from
+//      memory in their own layouts; a lane ends with four consecutive outputs of one token.
+//   4. a token's rows are added in the order its experts were chosen: by the norm that reads them next
+//      (it is handed the list `where`), or by moe_combine.
+#include "common.h"
+#include "tinyinfer_kernels.h"
+
+TI_ERROR_API
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+union Frag8 {
+  uint4 u;
+  bf16x8 v;
+};
+
+#define MOE_TILE 64          // rows (pairs) of a tile
+#define MOE_MAX_E 1024
+
+// meta int32: [0] number of tiles, [1 .. E + 1] offsets of the experts' runs, then E cursors, then tiles [max][3] =
+// (expert, first row, rows).  One workgroup.
+__global__ void __launch_bounds__(1024)
+moe_group_kernel(const int* __restrict__ ids, int n_pairs, int E, int* __restrict__ meta) {
+  __shared__ int count[MOE_MAX_E];
+  __shared__ int first_tile[MOE_MAX_E + 1];
+  for (int e = threadIdx.x; e < E; e += 1024) count[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_pairs; i += 1024) atomicAdd(&count[ids[i]], 1);
+  __syncthreads();
+  int* offsets = meta + 1;
+  int* cursors = meta + 1 + E + 1;
+  int* tiles = cursors + E;
+  if (threadIdx.x == 0) {
+    int at = 0, t = 0;
+    for (int e = 0; e < E; ++e) {
+      offsets[e] = at;
+      first_tile[e] = t;
+      at += count[e];
+      t += (count[e] + MOE_TILE - 1) / MOE_TILE;
+    }
+    offsets[E] = at;
+    first_tile[E] = t;
+    meta[0] = t;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 1024) {
+    cursors[e] = 0;
+    const int n = count[e], t0 = first_tile[e];
+    for (int k = 0; k * MOE_TILE < n; ++k) {
+      tiles[3 * (t0 + k)] = e;
+      tiles[3 * (t0 + k) + 1] = offsets[e] + k * MOE_TILE;
+      tiles[3 * (t0 + k) + 2] = min(MOE_TILE, n - k * MOE_TILE);
+    }
+  }
+}
+
+// a workgroup per pair: where[pair] = its row; rows[row] = bf16(s h[token]) (or h itself where the score scales the output)
+__global__ void __launch_bounds__(128)
+moe_place_kernel(const bf16_t* __restrict__ h, const int* __restrict__ ids, const float* __restrict__ wts, int* __restrict__ meta,
+                 int E, int top, int W, int scale_input, int* __restrict__ where, bf16_t* __restrict__ rows) {
+  __shared__ int s_row;
+  const int pair = blockIdx.x, m = pair / top;
+  if (threadIdx.x == 0) {
+    const int e = ids[pair];
+    const int r = meta[1 + e] + atomicAdd(&meta[1 + E + 1 + e], 1);
+    where[pair] = r;
+    s_row = r;
+  }
+  __syncthreads();
+  const float s = scale_input ? wts[pair] : 1.f;
+  const bf16_t* src = h + (size_t)m * W;
+  bf16_t* dst = rows + (size_t)s_row * W;
+  for (int c = threadIdx.x * 8; c < W; c += 128 * 8) {      // W is a multiple of 32
+    const uint4 a = *reinterpret_cast<const uint4*>(src + c);
+    const unsigned w[4] = {a.x, a.y, a.z, a.w};
+    unsigned o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = pack_bf16x2(__uint_as_float(w[i] << 16) * s, __uint_as_float(w[i] & 0xffff0000u) * s);
+    *reinterpret_cast<uint4*>(dst + c) = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
+// out[row][n] (op)= sum_k rows[row][k] w[e][n][k] over the tiles.  A workgroup: one tile of 64 rows x 128 outputs; wavefront v
+// the outputs 32 v .. 32 v + 31 of it (two blocks of 16) against the four blocks of 16 rows.  EPI 0: relu^2, bfloat16; 1: 32-bit.
+template <int EPI>
+__global__ void __launch_bounds__(256)
+moe_grouped_kernel(const bf16_t* __restrict__ rows, const bf16_t* __restrict__ w, const int* __restrict__ meta, int E, void* __restrict__ out,
+                   int N, int K) {
+  const int n_tiles = meta[0];
+  if ((int)blockIdx.x >= n_tiles) return;
+  const int* tile = meta + 1 + E + 1 + E + 3 * blockIdx.x;
+  const int e = tile[0], row0 = tile[1], n_rows = tile[2];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r16 = lane & 15, quad = lane >> 4;
+  const int n0 = blockIdx.y * 128 + wave * 32;
+  if (n0 >= N) return;
+  // operands: lane (r16, quad) holds 8 consecutive k of row r16 of its block, from k = 8 quad on
+  const bf16_t* wa[2];
+  const bf16_t* tb[4];
+#pragma unroll
+  for (int a = 0; a < 2; ++a) wa[a] = w + ((size_t)e * N + min(n0 + 16 * a + r16, N - 1)) * K + quad * 8;
+#pragma unroll
+  for (int b = 0; b < 4; ++b) tb[b] = rows + (size_t)(row0 + min(16 * b + r16, n_rows - 1)) * K + quad * 8;
+  floatx4 acc[2][4];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) acc[a][b] = floatx4{0.f, 0.f, 0.f, 0.f};
+  Frag8 fa[2][2], fb[2][4];
+  auto load = [&](int k, int s) {
+#pragma unroll
+    for (int a = 0; a < 2; ++a) fa[s][a].u = *reinterpret_cast<const uint4*>(wa[a] + k);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) fb[s][b].u = *reinterpret_cast<const uint4*>(tb[b] + k);
+  };
+  auto multiply = [&](int s) {
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[s][a].v, fb[s][b].v, acc[a][b], 0, 0, 0);
+  };
+  load(0, 0);
+  for (int k = 0; k < K; k += 64) {       // K is a multiple of 32
+    if (k + 32 < K) load(k + 32, 1);
+    multiply(0);
+    if (k + 32 >= K) break;
+    if (k + 64 < K) load(k + 64, 0);
+    multiply(1);
+  }
+  // lane: outputs n0 + 16 a + 4 quad + i of row 16 b + r16
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int r = 16 * b + r16;
+    if (r >= n_rows) continue;
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      const int n = n0 + 16 * a + 4 * quad;
+      if (n >= N) continue;                 // N is a multiple of 4
+      const floatx4 v = acc[a][b];
+      if (EPI == 0) {
+        float z[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          z[i] = fmaxf(v[i], 0.f);
+          z[i] *= z[i];
+        }
+        *reinterpret_cast<uint2*>((bf16_t*)out + (size_t)(row0 + r) * N + n) = make_uint2(pack_bf16x2(z[0], z[1]), pack_bf16x2(z[2], z[3]));
+      } else {
+        *reinterpret_cast<float4*>((float*)out + (size_t)(row0 + r) * N + n) = make_float4(v[0], v[1], v[2], v[3]);
+      }
+    }
+  }
+}
+
+// y[m] = sum_k out[where[m top + k]], k ascending
+__global__ void moe_combine_kernel(const float* __restrict__ out, const int* __restrict__ where, float* __restrict__ y, int W, int top) {
+  const int m = blockIdx.x;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float v = 0.f;
+    for (int k = 0; k < top; ++k) v += out[(size_t)where[m * top + k] * W + c];
+    y[(size_t)m * W + c] = v;
+  }
+}
+
+extern "C" long ti_moe_grouped_meta_ints(int n_pairs, int E) { return 1 + (E + 1) + E + 3L * ((n_pairs + MOE_TILE - 1) / MOE_TILE + E); }
+
+// h bf16 [M, W]; ids, wts [M top]; up [E][F][W], down [E][W][F] bf16.  Scratch: meta int32 [ti_moe_grouped_meta_ints],
+// where int32 [M top], rows bf16 [M top][W], act bf16 [M top][F], out f32 [M top][W].  y (may be null): the tokens' sums;
+// without it the caller adds the rows out[where[m top + k]] itself.  3: sizes not served (W, F multiples of 32, E <= 1024).
+extern "C" int ti_moe_experts_grouped_bf16(const void* h, const int* ids, const float* wts, const void* up, const void* down,
+                                           int* meta, int* where, void* rows, void* act, float* out, float* y, int M, int W, int F,
+                                           int E, int top, int scale_input, hipStream_t stream) {
+  if (W % 32 || F % 32 || E > MOE_MAX_E || !scale_input) {
+    ti_set_error("moe_experts (grouped): W=%d, F=%d, %d experts are not served", W, F, E);
+    return 3;
+  }
+  TI_REQUIRE(M >= 0 && top > 0 && E > 0, "moe_experts (grouped): bad sizes");
+  if (M == 0) return 0;
+  const int n_pairs = M * top;
+  const int max_tiles = (n_pairs + MOE_TILE - 1) / MOE_TILE + E;
+  moe_group_kernel<<<1, 1024, 0, stream>>>(ids, n_pairs, E, meta);
+  moe_place_kernel<<<n_pairs, 128, 0, stream>>>((const bf16_t*)h, ids, wts, meta, E, top, W, scale_input, where, (bf16_t*)rows);
+  moe_grouped_kernel<0><<<dim3(max_tiles, (F + 127) / 128), 256, 0, stream>>>((const bf16_t*)rows, (const bf16_t*)up, meta, E, act, F, W);
+  moe_grouped_kernel<1><<<dim3(max_tiles, (W + 127) / 128), 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, meta, E, out, W, F);
+  if (y) moe_combine_kernel<<<M, 256, 0, stream>>>(out, where, y, W, top);
+  TI_LAUNCH_CHECK();
+  return 0;
+}

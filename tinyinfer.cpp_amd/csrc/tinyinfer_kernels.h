@@ -181,9 +181,19 @@ int ti_diff_attention_rows_bf16(const void* q, const void* pool, const int* tabl
 int ti_moe_route(int dtype, const void* h, const float* router, int* ids, float* wts, int M, int W, int E, int top,
                  int score_kind, int renormalize, hipStream_t stream);
 // y f32 [M, W] = sum_k down[e_k] relu(up[e_k] (s_k h))^2 (scale_input) or sum_k s_k down[e_k] relu(up[e_k] h)^2;
-// up [E][F][W], down [E][W][F] in the dtype of h
-int ti_moe_experts_rows(int dtype, const void* h, const int* ids, const float* wts, const void* up, const void* down, float* y,
-                        int M, int W, int F, int top, int scale_input, hipStream_t stream);
+// up [E][F][W], down [E][W][F] in the dtype of h; act: scratch of that dtype, [M top][F].  An output a wavefront: steps of
+// few tokens, and float32
+int ti_moe_experts_rows(int dtype, const void* h, const int* ids, const float* wts, const void* up, const void* down, void* act,
+                        float* y, int M, int W, int F, int top, int scale_input, hipStream_t stream);
+
+// ---- libti_moe_bf16: the experts for steps of many tokens, on the matrix cores: the (token, expert) pairs are laid out expert
+// by expert in tiles of 64 rows and both products run over the tiles.  Scratch: meta int32 [ti_moe_grouped_meta_ints(M top, E)],
+// where int32 [M top] (the row of every pair), rows bf16 [M top][W], act bf16 [M top][F], out f32 [M top][W].  y (may be
+// null): the tokens' sums; without it the caller adds the rows out[where[m top + k]] in ascending k.  3: sizes not served
+long ti_moe_grouped_meta_ints(int n_pairs, int E);
+int ti_moe_experts_grouped_bf16(const void* h, const int* ids, const float* wts, const void* up, const void* down, int* meta,
+                                int* where, void* rows, void* act, float* out, float* y, int M, int W, int F, int E, int top,
+                                int scale_input, hipStream_t stream);
 
 // ---- libti_attention_bf16: the same on the matrix cores (head sizes 32, 64, 128; pages of 16 n rows)
 // rows of single tokens; n_splits > 1 needs part_o f32 [n_rows, n_head, n_splits, hd] and part_ml f32

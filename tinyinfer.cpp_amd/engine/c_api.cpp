@@ -1299,7 +1299,7 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
     ops.moe_route(arg(0), arg(1), arg(2), arg(3), (int)num(0), (Ops::RouterScore)(int)num(1), num(2) != 0);
   } else if (op == "moe_experts") {
     // h, ids, wts, up, down, y; experts, scale_input
-    ops.moe_experts(arg(0), arg(1), arg(2), arg(3), arg(4), arg(5), (int)num(0), num(1) != 0);
+    ops.moe_experts(arg(0), arg(1), arg(2), arg(3), arg(4), arg(5), (int)num(0), num(1) != 0, workspace_of(&ops));
   } else if (op == "argmax") {
     ops.argmax(arg(0), arg(1).ptr<int>());
   } else if (op == "sample") {

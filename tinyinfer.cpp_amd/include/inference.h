@@ -379,9 +379,12 @@ class Ops {
   void moe_route(const Tensor& h, const Tensor& router, const Tensor& ids, const Tensor& wts, int top, RouterScore score,
                  bool renormalize);
   // y f32 [M, W] = sum over a token's experts of down_e relu(up_e h)^2, the weight on the expert's input or output;
-  // up [E F, W], down [E W, F]
+  // up [E F, W], down [E W, F]; scratch comes from `ws`.  With `rows` (and bfloat16, many tokens, sizes the matrix-core kernels
+  // take) y may stay unwritten: then rows->t is f32 [M top, W] and rows->gather device int32 [M][top]: row m of the result is
+  // the sum of the rows rows->t[gather[m][k]], k ascending, left to the norm that reads it (Ops::norm_residual)
+  struct GatheredRows { Tensor t; const int* gather = nullptr; int n_gather = 0; };
   void moe_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, const Tensor& up, const Tensor& down, const Tensor& y,
-                   int experts, bool scale_input);
+                   int experts, bool scale_input, Workspace& ws, GatheredRows* rows = nullptr);
   void argmax(const Tensor& logits, int* out);
   void sample(const Tensor& logits, const float* temperature, const int* top_k, const float* top_p, const float* uniform,
               int* out);
@@ -623,6 +626,13 @@ class FeedForwardPart : public Part { public: using Part::Part; const char* fami
   virtual void forward(StepContext& ctx, const Rows& h, const Tensor& x) = 0;
   virtual bool can_store() const { return false; }
   virtual void forward_store(StepContext& ctx, const Rows& h, const Tensor& y);
+  // as forward_store, but the part may leave the last sum to its reader: it returns rows whose sums (Ops::GatheredRows) are
+  // its output, for a norm that adds them while it reads (NormPart::forward_add).  Default: forward_store, rows.t = y
+  virtual void forward_rows(StepContext& ctx, const Rows& h, const Tensor& y, Ops::GatheredRows& rows) {
+    forward_store(ctx, h, y);
+    rows = Ops::GatheredRows();
+    rows.t = y;
+  }
   virtual bool takes_lazy_norm() const { return false; } };
 class BlockPart : public Part { public: using Part::Part; const char* family() const override { return "block"; }
   virtual void forward(StepContext& ctx, const Tensor& x) = 0; };

@@ -396,7 +396,8 @@ class Ops:
 
     def moe_experts(self, h, ids, wts, up, down, y, experts, scale_input=True):
         """y f32 [M, W] = sum over a token's experts; up [experts F, W], down [experts W, F]."""
-        self._call("moe_experts", [h, ids, wts, up, down, y], [experts, int(bool(scale_input))])
+        libs = ["moe"] + (["moe_bf16"] if h.dtype == native.torch().bfloat16 else [])
+        self._call("moe_experts", [h, ids, wts, up, down, y], [experts, int(bool(scale_input))], libs=libs)
 
     def argmax(self, logits, out):
         if out.dtype != native.torch().int32 or out.shape[0] < logits.shape[0]:

@@ -1115,7 +1115,7 @@ void Ops::moe_route(const Tensor& h, const Tensor& router, const Tensor& ids, co
 }
 
 void Ops::moe_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, const Tensor& up, const Tensor& down, const Tensor& y,
-                      int experts, bool scale_input) {
+                      int experts, bool scale_input, Workspace& ws, GatheredRows* rows) {
   TIMED("moe_experts " + dims(h) + " * " + dims(up));
   require(h.ndim == 2 && h.contiguous() && up.ndim == 2 && down.ndim == 2 && up.contiguous() && down.contiguous() &&
               up.dtype == h.dtype && down.dtype == h.dtype && experts > 0,
@@ -1128,12 +1128,38 @@ void Ops::moe_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, con
           "moe_experts: y " + y.describe() + " does not fit");
   require(ids.dtype == DType::I32 && wts.dtype == DType::F32 && ids.numel() == wts.numel() && (M == 0 || ids.numel() % M == 0),
           "moe_experts: ids and wts must be int32 / float32 [M, top]");
+  if (rows) *rows = GatheredRows();
   if (M == 0) return;
   const int top = (int)(ids.numel() / M);
+  const int64_t pairs = M * top;
+  // many tokens: the pairs grouped by expert, both products on the matrix cores
+  if (h.dtype == DType::BF16 && use.fast_gemm && pairs >= 128 && kernel_library_available("moe_bf16")) {
+    const long meta_ints = KERNEL("moe_bf16", ti_moe_grouped_meta_ints)((int)pairs, experts);
+    int* meta = (int*)ws.get("moe.meta", (size_t)meta_ints * 4);
+    Tensor where = ws.tensor("moe.where", DType::I32, {pairs});
+    Tensor sorted = ws.tensor("moe.rows", DType::BF16, {pairs, W});
+    Tensor act = ws.tensor("moe.act", DType::BF16, {pairs, F});
+    Tensor out = ws.tensor("moe.out", DType::F32, {pairs, W});
+    int rc = KERNEL("moe_bf16", ti_moe_experts_grouped_bf16)(h.data, (const int*)ids.data, (const float*)wts.data, up.data, down.data, meta,
+                                                             (int*)where.data, sorted.data, act.data, (float*)out.data,
+                                                             rows ? nullptr : (float*)y.data, (int)M, (int)W, (int)F, experts, top,
+                                                             scale_input ? 1 : 0, (hipStream_t)launch_stream());
+    if (rc == 0) {
+      took(rows ? "[mfma, grouped, sums left]" : "[mfma, grouped]");
+      if (rows) {
+        rows->t = out;
+        rows->gather = (const int*)where.data;
+        rows->n_gather = top;
+      }
+      return;
+    }
+    if (rc != 3) check("moe_bf16", rc, "moe_experts(grouped)");
+  }
   took("[rows]");
+  Tensor act = ws.tensor("moe.act", h.dtype, {pairs, F});
   int rc = KERNEL("moe", ti_moe_experts_rows)(code(h.dtype, "moe_experts"), h.data, (const int*)ids.data, (const float*)wts.data,
-                                              up.data, down.data, (float*)y.data, (int)M, (int)W, (int)F, top, scale_input ? 1 : 0,
-                                              (hipStream_t)launch_stream());
+                                              up.data, down.data, act.data, (float*)y.data, (int)M, (int)W, (int)F, top,
+                                              scale_input ? 1 : 0, (hipStream_t)launch_stream());
   check("moe", rc, "moe_experts");
 }
 

@@ -1488,9 +1488,8 @@ class MoE final : public FeedForwardPart {
     if (experts < 1 || experts > 1024) throw ConfigError("moe: " + std::to_string(experts) + " experts are not served (1 to 1024)");
     if (top < 1 || top > experts || top > 64)
       throw ConfigError("moe: top " + std::to_string(top) + " must lie between 1 and the number of experts (and at most 64)");
-    if ((hidden + intermediate) * 4 > 64 * 1024)
-      throw ConfigError("moe: a width of " + std::to_string(hidden) + " beside an expert size of " + std::to_string(intermediate) +
-                        " is not served (the rows of one token and expert must fit 64 KB)");
+    if (hidden * 4 > 64 * 1024)
+      throw ConfigError("moe: a width of " + std::to_string(hidden) + " is not served (a token's row must fit 64 KB)");
     const std::string act = p.has("activation") ? p.at("activation").as_string() : "relu2";
     if (act != "relu2") throw ConfigError("moe: activation '" + act + "' is not served (only 'relu2')");
     const std::string sc = p.has("score") ? p.at("score").as_string() : "sigmoid";
@@ -1532,13 +1531,19 @@ class MoE final : public FeedForwardPart {
     router.role = TensorNeed::Vector;
     w_router = src.fetch(n_router, router);
   }
-  void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override {
+  void run(StepContext& ctx, const Rows& h, const Tensor& y, Ops::GatheredRows* left) {
     const Tensor& rows = h.materialize(ctx.ops);
     const int64_t M = rows.shape[0];
     Tensor ids = ctx.buf("moe.ids", DType::I32, {M, (int64_t)top});
     Tensor wts = ctx.buf("moe.wts", DType::F32, {M, (int64_t)top});
     ctx.ops.moe_route(rows, w_router, ids, wts, top, score, renormalize);
-    ctx.ops.moe_experts(rows, ids, wts, w_up, w_down, y, experts, scale_input);
+    ctx.ops.moe_experts(rows, ids, wts, w_up, w_down, y, experts, scale_input, ctx.ws, left);
+  }
+  void forward_store(StepContext& ctx, const Rows& h, const Tensor& y) override { run(ctx, h, y, nullptr); }
+  // the sum over a token's experts may be left to the norm that reads the result
+  void forward_rows(StepContext& ctx, const Rows& h, const Tensor& y, Ops::GatheredRows& rows) override {
+    run(ctx, h, y, &rows);
+    if (!rows.t.defined()) rows.t = y;
   }
   void forward(StepContext& ctx, const Rows& h, const Tensor& x) override {
     Tensor y = ctx.buf("moe.y", DType::F32, {x.shape[0], hidden});
@@ -1607,8 +1612,9 @@ class PostNormBlock final : public BlockPart {
     mixer->forward_store(ctx, input(ctx, x), y);
     norm1->forward_add(ctx, y, x, true);
     if (!ffn) return;
-    ffn->forward_store(ctx, input(ctx, x), y);
-    norm2->forward_add(ctx, y, x, true);
+    Ops::GatheredRows rows;
+    ffn->forward_rows(ctx, input(ctx, x), y, rows);
+    norm2->forward_add(ctx, rows.t, x, true, rows.gather, rows.n_gather);
   }
   std::shared_ptr<NormPart> norm1, norm2;
   std::shared_ptr<MixerPart> mixer;
