@@ -65,6 +65,11 @@ def test_norm_into_the_residual(ops, H):
     ops.norm_residual(x, dev(src), dev(g), 1e-5, True, dev(gather, torch.int32))
     want = x0 + plain.rms_unit(src[gather[:, 0]] + src[gather[:, 1]], 1e-5) * g
     assert np.abs(f64(x) - want).max() < 3e-6
+    # a rounded copy of the new residual beside it
+    x, copy = dev(x0), torch.empty(5, H, device="cuda", dtype=torch.bfloat16)
+    ops.norm_residual(x, dev(y), dev(g), 1e-5, True, None, copy)
+    assert np.abs(f64(x) - (x0 + normed)).max() < 3e-6
+    assert torch.equal(copy, x.to(torch.bfloat16))
 
 
 def test_round_rows_and_scale(ops):
@@ -117,6 +122,44 @@ def test_short_conv_carries_its_state_through_any_cut(ops, K, C):
         results.append((a, b))
     for a, b in results[1:]:                                # the same bits however the rows were cut
         assert np.array_equal(a, results[0][0]) and np.array_equal(b, results[0][1])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_convolution_inside_the_preparation_gives_the_same_bits(ops, dtype):
+    """The projections of two requests in several cuts: convolution, then preparation, against the preparation that takes the
+    convolution in.  Queries and pages hold the same bits, and so does the state that is left."""
+    rng = np.random.default_rng(5)
+    heads, kv, dk, dv, P, K, T = 3, 1, 12, 20, 8, 4, 37
+    C = heads * 2 * dk + kv * (2 * dk + dv)
+    u = [rng.normal(size=(T, C)), rng.normal(size=(T, C))]
+    taps = dev(rng.normal(size=(C, K)))
+    qw, kw = dev(1.0 + rng.normal(size=dk) * 0.2), dev(1.0 + rng.normal(size=dk) * 0.2)
+    inv = dev(np.array([50.0 ** (-2.0 * i / 8) for i in range(4)]))
+    table = dev(np.array([[4, 1, 7, 0, 9], [2, 8, 3, 6, 5]]), torch.int32)
+    results = []
+    for inside in (False, True):
+        state = torch.zeros(3, K - 1, C, device="cuda")
+        pool = torch.zeros(10, kv, P, 2 * dk + dv, device="cuda", dtype=DT[dtype])
+        qs, at = [], 0
+        for n in (5, 1, 2, 1, 20, 3, 5):
+            rows = dev(np.concatenate([u[0][at:at + n], u[1][at:at + n]]))
+            entries = dev([[0, n, at, 2], [n, n, at, 0]], torch.int32)
+            entry_of = dev([0] * n + [1] * n, torch.int32)
+            pos = dev(list(range(at, at + n)) * 2, torch.int32)
+            q_out = torch.empty(2 * n, heads * 2 * dk, device="cuda", dtype=DT[dtype])
+            if inside:
+                ops.diff_qk_prep(rows, qw, kw, inv, None, pos, entry_of, table, pool, q_out, 1e-5, heads, kv, dk, dv, 8, 1.1,
+                                 taps=taps, state=state, entries=entries)
+            else:
+                mixed = torch.empty_like(rows)
+                ops.short_conv(rows, taps, state, entries, entry_of, pos, mixed)
+                ops.diff_qk_prep(mixed, qw, kw, inv, None, pos, entry_of, table, pool, q_out, 1e-5, heads, kv, dk, dv, 8, 1.1)
+            qs.append(q_out)
+            at += n
+        results.append((torch.cat(qs), pool, state))
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    assert results[0][2].abs().sum() > 0
 
 
 def paged(rng, n_tokens, P, extra_pages=3):

@@ -74,43 +74,75 @@ extern "C" int ti_short_conv(const float* u, const float* taps, float* state, co
 // first rot_dims entries are turned: entry i with entry i + rot_dims / 2 by the angle pos * inv_freq[i], cosine and
 // sine times `mag` (the table [table_len][rot_dims / 2][2] holds them ready for positions below table_len).
 // q goes to q_out (T) [M, n_head 2 dk], k and v into the page of the token's position.
-template <typename T>
+// CONV: the rows of qkv are what the projection left, and every channel first passes the short convolution above (taps,
+// state, entries, entry_of as in short_conv_kernel; the state itself is moved on by short_conv_state_kernel afterwards):
+// the same sums in the same order as the convolution on its own, so the same bits.
+template <typename T, bool CONV>
 __global__ void __launch_bounds__(256)
-diff_qk_prep_kernel(const float* __restrict__ qkv, const float* __restrict__ q_w, const float* __restrict__ k_w, float eps,
+diff_qk_prep_kernel(const float* __restrict__ qkv, const float* __restrict__ taps, const float* __restrict__ state,
+                    const int* __restrict__ entries, const int* __restrict__ entry_of, int K,
+                    const float* __restrict__ q_w, const float* __restrict__ k_w, float eps,
                     const float* __restrict__ inv_freq, const float* __restrict__ rope_table, int table_len, float mag,
                     int rot_dims, const int* __restrict__ pos, const int* __restrict__ slot, const int* __restrict__ table,
                     int table_stride, T* __restrict__ pool, T* __restrict__ q_out, int n_head, int n_kv, int dk, int dv, int P) {
+  __shared__ float s_unit[4][256];      // a wavefront's unit after the convolution (dk <= 256)
   const int m = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int p = pos[m];
   const int nq = n_head * 2 * dk, nk = n_kv * 2 * dk, nv = n_kv * dv;
-  const float* row = qkv + (size_t)m * (nq + nk + nv);
+  const int C = nq + nk + nv;
+  const float* row = qkv + (size_t)m * C;
+  int row0 = 0, start = 0;
+  const float* st_rows = nullptr;
+  if (CONV) {
+    const int e = entry_of[m];
+    row0 = entries[4 * e];
+    start = entries[4 * e + 2];
+    st_rows = state + (size_t)entries[4 * e + 3] * (K - 1) * C;
+  }
+  // channel c of this token behind the convolution (or as it is)
+  auto channel = [&](int c) {
+    if (!CONV) return row[c];
+    float acc = 0.f;
+    for (int j = 0; j < K; ++j) {
+      const int s = p - (K - 1) + j;
+      const float v = s >= start ? qkv[(size_t)(row0 + s - start) * C + c] : st_rows[(size_t)(s - start + K - 1) * C + c];
+      acc = fmaf(taps[(size_t)c * K + j], v, acc);
+    }
+    return acc;
+  };
   const int page = table[(size_t)slot[m] * table_stride + p / P];
   const int r = p % P;
   T* base = pool + (size_t)max(page, 0) * ((size_t)n_kv * P * (2 * dk + dv));
   const int half = rot_dims / 2;
   const int units = 2 * n_head + 2 * n_kv;
-  for (int u = wave; u < units; u += 4) {
+  float* unit = s_unit[wave];
+  // a wavefront's piece of work: a map of a head (norm, rotation), or 64 channels of v; four pieces a workgroup
+  const int u = blockIdx.y * 4 + wave;
+  if (u < units) {
     const bool is_q = u < 2 * n_head;
-    const float* src = row + (size_t)u * dk;          // q's units, then k's: the row holds them in this order
     const float* w = is_q ? q_w : k_w;
     float ss = 0.f;
-    for (int d = lane; d < dk; d += 64) ss = fmaf(src[d], src[d], ss);
+    for (int d = lane; d < dk; d += 64) {
+      const float v = channel(u * dk + d);          // q's units, then k's: the row holds them in this order
+      unit[d] = v;
+      ss = fmaf(v, v, ss);
+    }
     const float scale = 1.0f / sqrtf(group_sum<64>(ss) / (float)dk + eps);
     T* dst;
     if (is_q) {
       dst = q_out + (size_t)m * nq + (size_t)u * dk;
     } else {
-      if (page < 0) continue;      // the host reserves pages first; never write astray
+      if (page < 0) return;        // the host reserves pages first; never write astray
       const int ku = u - 2 * n_head;
       dst = base + ((size_t)(ku >> 1) * P + r) * (2 * dk) + (size_t)(ku & 1) * dk;
     }
     for (int d = lane; d < dk; d += 64) {
-      float v = src[d] * scale * (w ? w[d] : 1.f);
+      float v = unit[d] * scale * (w ? w[d] : 1.f);
       if (d < rot_dims) {
         const int i = d < half ? d : d - half;
         const int other = d < half ? d + half : d - half;
-        const float o = src[other] * scale * (w ? w[other] : 1.f);
+        const float o = unit[other] * scale * (w ? w[other] : 1.f);
         float c, s;
         if (rope_table && p < table_len) {
           c = rope_table[((size_t)p * half + i) * 2];
@@ -124,35 +156,50 @@ diff_qk_prep_kernel(const float* __restrict__ qkv, const float* __restrict__ q_w
       }
       st<T>(dst + d, v);
     }
+    return;
   }
-  if (page < 0) return;
+  const int e = (u - units) * 64 + lane;
+  if (page < 0 || e >= nv) return;
   T* vbase = base + (size_t)n_kv * P * 2 * dk;
-  for (int e = threadIdx.x; e < nv; e += 256) {
-    const int h = e / dv, d = e % dv;
-    st<T>(vbase + ((size_t)h * dv + d) * P + r, row[nq + nk + e]);
-  }
+  const int h = e / dv, d = e % dv;
+  st<T>(vbase + ((size_t)h * dv + d) * P + r, channel(nq + nk + e));
 }
 
-extern "C" int ti_diff_qk_prep(int dtype, const float* qkv, const float* q_w, const float* k_w, float eps,
-                               const float* inv_freq, const float* rope_table, int table_len, float mag, int rot_dims,
-                               const int* pos, const int* slot, const int* table, int table_stride, void* pool, void* q_out,
-                               int M, int n_head, int n_kv, int dk, int dv, int page_size, hipStream_t stream) {
-  TI_REQUIRE(n_head > 0 && n_kv > 0 && dk > 0 && dv > 0 && page_size > 0 && table_stride > 0,
+// taps f32 [C][K] (null: no convolution), state f32 [slots][K - 1][C], entries int32 [n_entries][4], entry_of int32 [M]
+extern "C" int ti_diff_qk_prep(int dtype, const float* qkv, const float* taps, float* state, const int* entries, int n_entries,
+                               const int* entry_of, int K, const float* q_w, const float* k_w, float eps, const float* inv_freq,
+                               const float* rope_table, int table_len, float mag, int rot_dims, const int* pos, const int* slot,
+                               const int* table, int table_stride, void* pool, void* q_out, int M, int n_head, int n_kv, int dk,
+                               int dv, int page_size, hipStream_t stream) {
+  TI_REQUIRE(n_head > 0 && n_kv > 0 && dk > 0 && dk <= 256 && dv > 0 && page_size > 0 && table_stride > 0,
              "diff_qk_prep: bad sizes heads=%d kv_heads=%d dk=%d dv=%d page=%d", n_head, n_kv, dk, dv, page_size);
   TI_REQUIRE(rot_dims >= 0 && rot_dims <= dk && rot_dims % 2 == 0 && (rot_dims == 0 || inv_freq),
              "diff_qk_prep: %d rotated entries do not fit a key of %d", rot_dims, dk);
+  TI_REQUIRE(!taps || (K >= 1 && entries && entry_of && (K == 1 || state)), "diff_qk_prep: the convolution needs taps, entries and a state");
   if (M == 0) return 0;
-  if (dtype == TI_F32)
-    diff_qk_prep_kernel<float><<<M, 256, 0, stream>>>(qkv, q_w, k_w, eps, inv_freq, rope_table, table_len, mag, rot_dims, pos,
-                                                      slot, table, table_stride, (float*)pool, (float*)q_out, n_head, n_kv, dk,
-                                                      dv, page_size);
-  else if (dtype == TI_BF16)
-    diff_qk_prep_kernel<bf16_t><<<M, 256, 0, stream>>>(qkv, q_w, k_w, eps, inv_freq, rope_table, table_len, mag, rot_dims, pos,
-                                                       slot, table, table_stride, (bf16_t*)pool, (bf16_t*)q_out, n_head, n_kv,
-                                                       dk, dv, page_size);
-  else
+  const int pieces = 2 * n_head + 2 * n_kv + (n_kv * dv + 63) / 64;
+  const dim3 grid(M, (pieces + 3) / 4);
+#define DQ_LAUNCH(T, CONV)                                                                                                          \
+  diff_qk_prep_kernel<T, CONV><<<grid, 256, 0, stream>>>(qkv, taps, state, entries, entry_of, K, q_w, k_w, eps, inv_freq, rope_table,  \
+                                                         table_len, mag, rot_dims, pos, slot, table, table_stride, (T*)pool,       \
+                                                         (T*)q_out, n_head, n_kv, dk, dv, page_size)
+  if (dtype == TI_F32) {
+    if (taps) DQ_LAUNCH(float, true);
+    else DQ_LAUNCH(float, false);
+  } else if (dtype == TI_BF16) {
+    if (taps) DQ_LAUNCH(bf16_t, true);
+    else DQ_LAUNCH(bf16_t, false);
+  } else {
     TI_REQUIRE(false, "diff_qk_prep: unknown dtype %d", dtype);
+  }
+#undef DQ_LAUNCH
   TI_LAUNCH_CHECK();
+  if (taps && K > 1 && n_entries > 0) {
+    const int C = n_head * 2 * dk + n_kv * (2 * dk + dv);
+    dim3 grid(n_entries, (C + 255) / 256 < 64 ? (C + 255) / 256 : 64);
+    short_conv_state_kernel<<<grid, 256, 0, stream>>>(qkv, state, entries, C, K);
+    TI_LAUNCH_CHECK();
+  }
   return 0;
 }
 

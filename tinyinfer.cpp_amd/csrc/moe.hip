@@ -16,11 +16,50 @@ TI_ERROR_API
 #define MOE_SIGMOID 0
 #define MOE_SOFTMAX 1
 
+template <typename T> struct Piece;
+template <> struct Piece<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ void load(const float* p, float* v) {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+  }
+};
+template <> struct Piece<bf16_t> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void load(const bf16_t* p, float* v) {
+    const uint4 a = *reinterpret_cast<const uint4*>(p);
+    const unsigned w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(w[i] << 16);
+      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+};
+
+// the wavefront's share of a . b over n elements: a in LDS or memory as floats through `fa`, b a row of the weight
+template <typename T, bool VEC, class FA>
+__device__ __forceinline__ float wave_dot(FA fa, const T* __restrict__ b, int n, int lane) {
+  float z = 0.f;
+  if (VEC) {
+    constexpr int N = Piece<T>::N;
+    for (int c = lane * N; c < n; c += 64 * N) {
+      float v[N];
+      Piece<T>::load(b + c, v);
+#pragma unroll
+      for (int i = 0; i < N; ++i) z = fmaf(fa(c + i), v[i], z);
+    }
+  } else {
+    for (int c = lane; c < n; c += 64) z = fmaf(fa(c), ld<T>(b + c), z);
+  }
+  return group_sum<64>(z);
+}
+
 // ------------------------------------------------------------ router
-// A workgroup per token.  Logits: wavefront w takes experts w, w + 4, ...; lanes share a row of the router
-// (lane l the entries l, l + 64, ... in ascending order, then a butterfly).  Choice: the first wavefront
+// A workgroup per token.  Logits: wavefront w takes experts w, w + 4, ...; lanes share the token's row in pieces of
+// 16 bytes (lane l the pieces l, l + 64, ... in ascending order, then a butterfly).  Choice: the first wavefront
 // holds the scores (lane l the experts l, l + 64, ...) and takes the largest `top` times.
-template <typename T>
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(256)
 moe_route_kernel(const T* __restrict__ h, const float* __restrict__ router, int* __restrict__ ids, float* __restrict__ wts,
                  int W, int E, int top, int score_kind, int renormalize) {
@@ -30,10 +69,7 @@ moe_route_kernel(const T* __restrict__ h, const float* __restrict__ router, int*
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const T* row = h + (size_t)m * W;
   for (int e = wave; e < E; e += 4) {
-    const float* r = router + (size_t)e * W;
-    float z = 0.f;
-    for (int c = lane; c < W; c += 64) z = fmaf(ld<T>(row + c), r[c], z);
-    z = group_sum<64>(z);
+    const float z = wave_dot<T, VEC>([&](int c) { return router[(size_t)e * W + c]; }, row, W, lane);
     if (lane == 0) s_score[e] = z;
   }
   __syncthreads();
@@ -89,9 +125,19 @@ extern "C" int ti_moe_route(int dtype, const void* h, const float* router, int* 
              MOE_MAX_TOP);
   TI_REQUIRE(score_kind == MOE_SIGMOID || score_kind == MOE_SOFTMAX, "moe_route: unknown score kind %d", score_kind);
   if (M == 0) return 0;
-  if (dtype == TI_F32) moe_route_kernel<float><<<M, 256, 0, stream>>>((const float*)h, router, ids, wts, W, E, top, score_kind, renormalize);
-  else if (dtype == TI_BF16) moe_route_kernel<bf16_t><<<M, 256, 0, stream>>>((const bf16_t*)h, router, ids, wts, W, E, top, score_kind, renormalize);
-  else TI_REQUIRE(false, "moe_route: unknown dtype %d", dtype);
+  const int piece = dtype == TI_F32 ? 4 : 8;
+  const bool vec = W % piece == 0 && ((uintptr_t)h & 15) == 0;
+#define MOE_ROUTE(T, V) moe_route_kernel<T, V><<<M, 256, 0, stream>>>((const T*)h, router, ids, wts, W, E, top, score_kind, renormalize)
+  if (dtype == TI_F32) {
+    if (vec) MOE_ROUTE(float, true);
+    else MOE_ROUTE(float, false);
+  } else if (dtype == TI_BF16) {
+    if (vec) MOE_ROUTE(bf16_t, true);
+    else MOE_ROUTE(bf16_t, false);
+  } else {
+    TI_REQUIRE(false, "moe_route: unknown dtype %d", dtype);
+  }
+#undef MOE_ROUTE
   TI_LAUNCH_CHECK();
   return 0;
 }
@@ -101,45 +147,6 @@ extern "C" int ti_moe_route(int dtype, const void* h, const float* router, int* 
 // token m and chosen expert k; then y[m][c] = sum_k down[e_k][c] . act[(m, k)], k ascending.  A wavefront owns ROWS outputs;
 // its lanes share a row of the weight in pieces of 16 bytes (lane l the pieces l, l + 64, ... in ascending order, then a
 // butterfly): the order of every sum is fixed, whatever else the step holds.
-template <typename T> struct Piece;
-template <> struct Piece<float> {
-  static constexpr int N = 4;
-  static __device__ __forceinline__ void load(const float* p, float* v) {
-    const float4 a = *reinterpret_cast<const float4*>(p);
-    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
-  }
-};
-template <> struct Piece<bf16_t> {
-  static constexpr int N = 8;
-  static __device__ __forceinline__ void load(const bf16_t* p, float* v) {
-    const uint4 a = *reinterpret_cast<const uint4*>(p);
-    const unsigned w[4] = {a.x, a.y, a.z, a.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      v[2 * i] = __uint_as_float(w[i] << 16);
-      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-    }
-  }
-};
-
-// the wavefront's share of a . b over n elements: a in LDS or memory as floats through `fa`, b a row of the weight
-template <typename T, bool VEC, class FA>
-__device__ __forceinline__ float wave_dot(FA fa, const T* __restrict__ b, int n, int lane) {
-  float z = 0.f;
-  if (VEC) {
-    constexpr int N = Piece<T>::N;
-    for (int c = lane * N; c < n; c += 64 * N) {
-      float v[N];
-      Piece<T>::load(b + c, v);
-#pragma unroll
-      for (int i = 0; i < N; ++i) z = fmaf(fa(c + i), v[i], z);
-    }
-  } else {
-    for (int c = lane; c < n; c += 64) z = fmaf(fa(c), ld<T>(b + c), z);
-  }
-  return group_sum<64>(z);
-}
-
 #define MOE_ROWS 4      // outputs a wavefront
 template <typename T, bool VEC>
 __global__ void __launch_bounds__(256)

@@ -87,8 +87,9 @@ moe_place_kernel(const bf16_t* __restrict__ h, const int* __restrict__ ids, cons
   }
 }
 
-// out[row][n] (op)= sum_k rows[row][k] w[e][n][k] over the tiles.  A workgroup: one tile of 64 rows x 128 outputs; wavefront v
-// the outputs 32 v .. 32 v + 31 of it (two blocks of 16) against the four blocks of 16 rows.  EPI 0: relu^2, bfloat16; 1: 32-bit.
+// out[row][n] (op)= sum_k rows[row][k] w[e][n][k] over the tiles.  A workgroup: one tile of 64 rows x 256 outputs; wavefront v
+// the outputs 64 v .. 64 v + 63 of it (four blocks of 16) against the four blocks of 16 rows: sixteen matrix instructions for
+// eight 16-byte loads a lane.  EPI 0: relu^2, bfloat16; 1: 32-bit.
 template <int EPI>
 __global__ void __launch_bounds__(256)
 moe_grouped_kernel(const bf16_t* __restrict__ rows, const bf16_t* __restrict__ w, const int* __restrict__ meta, int E, void* __restrict__ out,
@@ -99,30 +100,30 @@ moe_grouped_kernel(const bf16_t* __restrict__ rows, const bf16_t* __restrict__ w
   const int e = tile[0], row0 = tile[1], n_rows = tile[2];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r16 = lane & 15, quad = lane >> 4;
-  const int n0 = blockIdx.y * 128 + wave * 32;
+  const int n0 = blockIdx.y * 256 + wave * 64;
   if (n0 >= N) return;
   // operands: lane (r16, quad) holds 8 consecutive k of row r16 of its block, from k = 8 quad on
-  const bf16_t* wa[2];
+  const bf16_t* wa[4];
   const bf16_t* tb[4];
 #pragma unroll
-  for (int a = 0; a < 2; ++a) wa[a] = w + ((size_t)e * N + min(n0 + 16 * a + r16, N - 1)) * K + quad * 8;
+  for (int a = 0; a < 4; ++a) wa[a] = w + ((size_t)e * N + min(n0 + 16 * a + r16, N - 1)) * K + quad * 8;
 #pragma unroll
   for (int b = 0; b < 4; ++b) tb[b] = rows + (size_t)(row0 + min(16 * b + r16, n_rows - 1)) * K + quad * 8;
-  floatx4 acc[2][4];
+  floatx4 acc[4][4];
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+  for (int a = 0; a < 4; ++a)
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[a][b] = floatx4{0.f, 0.f, 0.f, 0.f};
-  Frag8 fa[2][2], fb[2][4];
+  Frag8 fa[2][4], fb[2][4];
   auto load = [&](int k, int s) {
 #pragma unroll
-    for (int a = 0; a < 2; ++a) fa[s][a].u = *reinterpret_cast<const uint4*>(wa[a] + k);
+    for (int a = 0; a < 4; ++a) fa[s][a].u = *reinterpret_cast<const uint4*>(wa[a] + k);
 #pragma unroll
     for (int b = 0; b < 4; ++b) fb[s][b].u = *reinterpret_cast<const uint4*>(tb[b] + k);
   };
   auto multiply = [&](int s) {
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int a = 0; a < 4; ++a)
 #pragma unroll
       for (int b = 0; b < 4; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[s][a].v, fb[s][b].v, acc[a][b], 0, 0, 0);
   };
@@ -140,7 +141,7 @@ moe_grouped_kernel(const bf16_t* __restrict__ rows, const bf16_t* __restrict__ w
     const int r = 16 * b + r16;
     if (r >= n_rows) continue;
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
+    for (int a = 0; a < 4; ++a) {
       const int n = n0 + 16 * a + 4 * quad;
       if (n >= N) continue;                 // N is a multiple of 4
       const floatx4 v = acc[a][b];
@@ -187,8 +188,8 @@ extern "C" int ti_moe_experts_grouped_bf16(const void* h, const int* ids, const 
   const int max_tiles = (n_pairs + MOE_TILE - 1) / MOE_TILE + E;
   moe_group_kernel<<<1, 1024, 0, stream>>>(ids, n_pairs, E, meta);
   moe_place_kernel<<<n_pairs, 128, 0, stream>>>((const bf16_t*)h, ids, wts, meta, E, top, W, scale_input, where, (bf16_t*)rows);
-  moe_grouped_kernel<0><<<dim3(max_tiles, (F + 127) / 128), 256, 0, stream>>>((const bf16_t*)rows, (const bf16_t*)up, meta, E, act, F, W);
-  moe_grouped_kernel<1><<<dim3(max_tiles, (W + 127) / 128), 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, meta, E, out, W, F);
+  moe_grouped_kernel<0><<<dim3(max_tiles, (F + 255) / 256), 256, 0, stream>>>((const bf16_t*)rows, (const bf16_t*)up, meta, E, act, F, W);
+  moe_grouped_kernel<1><<<dim3(max_tiles, (W + 255) / 256), 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, meta, E, out, W, F);
   if (y) moe_combine_kernel<<<M, 256, 0, stream>>>(out, where, y, W, top);
   TI_LAUNCH_CHECK();
   return 0;

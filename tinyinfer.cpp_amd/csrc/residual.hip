@@ -10,9 +10,11 @@ TI_ERROR_API
 // n_gather rows y[gather[m n_gather + k]] in ascending k (the rows a token's experts left).
 // A workgroup per row; each thread owns the elements t, t + 256, ... in both passes, so y and x may be
 // the same memory.  The sum of squares: per thread in ascending order, then block_sum (fixed order).
+// RT: also `rounded` (RT) [M][H] = the new x rounded, for the product that reads the residual next.
+template <typename RT>
 __global__ void __launch_bounds__(256)
 norm_residual_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ g,
-                     const int* __restrict__ gather, int n_gather, int H, float eps, int accumulate) {
+                     const int* __restrict__ gather, int n_gather, int H, float eps, int accumulate, RT* __restrict__ rounded) {
   __shared__ float red[4];
   const int m = blockIdx.x;
   auto value = [&](int i) {
@@ -31,15 +33,21 @@ norm_residual_kernel(float* __restrict__ x, const float* __restrict__ y, const f
   float* row = x + (size_t)m * H;
   for (int i = threadIdx.x; i < H; i += 256) {
     const float v = value(i) * scale * g[i];
-    row[i] = accumulate ? row[i] + v : v;
+    const float now = accumulate ? row[i] + v : v;
+    row[i] = now;
+    if (rounded) st<RT>(rounded + (size_t)m * H + i, now);
   }
 }
 
 extern "C" int ti_norm_residual(float* x, const float* y, const float* g, const int* gather, int n_gather, int M, int H,
-                                float eps, int accumulate, hipStream_t stream) {
+                                float eps, int accumulate, void* rounded, int rounded_dtype, hipStream_t stream) {
   TI_REQUIRE(M >= 0 && H > 0 && (!gather || n_gather > 0), "norm_residual: bad sizes M=%d H=%d gather=%d", M, H, n_gather);
+  TI_REQUIRE(!rounded || rounded_dtype == TI_F32 || rounded_dtype == TI_BF16, "norm_residual: unknown dtype %d", rounded_dtype);
   if (M == 0) return 0;
-  norm_residual_kernel<<<M, 256, 0, stream>>>(x, y, g, gather, n_gather, H, eps, accumulate);
+  if (rounded && rounded_dtype == TI_BF16)
+    norm_residual_kernel<bf16_t><<<M, 256, 0, stream>>>(x, y, g, gather, n_gather, H, eps, accumulate, (bf16_t*)rounded);
+  else
+    norm_residual_kernel<float><<<M, 256, 0, stream>>>(x, y, g, gather, n_gather, H, eps, accumulate, (float*)rounded);
   TI_LAUNCH_CHECK();
   return 0;
 }

@@ -134,9 +134,10 @@ int ti_gated_head_norm(int out_dtype, const float* o, const float* gate, int ld,
 
 // ---- libti_residual: layers that norm what a sublayer returns
 // x[m] (+)= y'[m] / sqrt(mean(y'[m]^2) + eps) * g; y'[m] = y[m], or with `gather` (int32 [M][n_gather]) the sum of
-// the rows y[gather[m][k]] in ascending k.  accumulate 0: x is overwritten (y may be x itself)
+// the rows y[gather[m][k]] in ascending k.  accumulate 0: x is overwritten (y may be x itself).  rounded (may be null):
+// [M][H] of rounded_dtype, the new x rounded for the product that reads it next
 int ti_norm_residual(float* x, const float* y, const float* g, const int* gather, int n_gather, int M, int H, float eps,
-                     int accumulate, hipStream_t stream);
+                     int accumulate, void* rounded, int rounded_dtype, hipStream_t stream);
 // out = x rounded to out_dtype
 int ti_round_rows(int out_dtype, const float* x, void* out, long n, hipStream_t stream);
 // x *= s
@@ -152,7 +153,10 @@ int ti_short_conv(const float* u, const float* taps, float* state, const int* en
 // norm with the weights q_w / k_w [dk] (may be null), rotation of the first rot_dims entries (entry i with entry
 // i + rot_dims / 2; cos and sin times mag; rope_table [table_len][rot_dims / 2][2] may be null), q to q_out, k and v
 // into pages K [n_kv][P][2 dk] | V [n_kv][dv][P]
-int ti_diff_qk_prep(int dtype, const float* qkv, const float* q_w, const float* k_w, float eps, const float* inv_freq,
+// With taps f32 [C][K] (C the width of qkv; null: none) every channel first passes the short convolution of ti_short_conv,
+// in the same kernel (state, entries, entry_of as there; the state is moved on afterwards): the same bits as the two calls
+int ti_diff_qk_prep(int dtype, const float* qkv, const float* taps, float* state, const int* entries, int n_entries,
+                    const int* entry_of, int K, const float* q_w, const float* k_w, float eps, const float* inv_freq,
                     const float* rope_table, int table_len, float mag, int rot_dims, const int* pos, const int* slot,
                     const int* table, int table_stride, void* pool, void* q_out, int M, int n_head, int n_kv, int dk, int dv,
                     int page_size, hipStream_t stream);

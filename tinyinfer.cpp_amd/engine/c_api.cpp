@@ -1259,9 +1259,11 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
     // o, proj, w, out; gate column, eps, heads, dv
     ops.gated_head_norm(arg(0), arg(1), (int)num(0), arg(2), (float)num(1), arg(3), (int)num(2), (int)num(3));
   } else if (op == "norm_residual") {
-    // x, y, gain, gather [M, n] (may be absent); eps, accumulate
+    // x, y, gain, gather [M, n] (may be absent), rounded copy (may be absent); eps, accumulate
     const bool g = n_t > 3 && arg(3).defined();
-    ops.norm_residual(arg(0), arg(1), arg(2), (float)num(0), num(1) != 0, g ? iptr(3) : nullptr, g ? (int)arg(3).shape[1] : 0);
+    const bool r = n_t > 4 && arg(4).defined();
+    ops.norm_residual(arg(0), arg(1), arg(2), (float)num(0), num(1) != 0, g ? iptr(3) : nullptr, g ? (int)arg(3).shape[1] : 0,
+                      r ? &arg(4) : nullptr);
   } else if (op == "round_rows") {
     ops.round_rows(arg(0), arg(1));
   } else if (op == "scale") {
@@ -1270,12 +1272,22 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
     // u, taps, state, entries [R, 4], entry of every row, positions, out
     ops.short_conv(arg(0), arg(1), arg(2), iptr(3), (int)arg(3).shape[0], iptr(4), iptr(5), arg(6));
   } else if (op == "diff_qk_prep") {
-    // qkv, q_w, k_w, inv_freq, rope_table, positions, slots, table, pool, q_out; eps, heads, kv_heads, dk, dv, rotated entries, mag
+    // qkv, q_w, k_w, inv_freq, rope_table, positions, slots, table, pool, q_out, [taps, state, entries [R, 4]: the short
+    // convolution inside]; eps, heads, kv_heads, dk, dv, rotated entries, mag
     Ops::Rotation r = rotation(3, 4);
     r.dims = (int)num(5);
     r.mag = (float)num(6);
+    Ops::ShortConv conv;
+    const bool with_conv = n_t > 12 && arg(10).defined();
+    if (with_conv) {
+      conv.taps = arg(10);
+      conv.state = arg(11);
+      conv.entry_meta = iptr(12);
+      conv.n_entries = (int)arg(12).shape[0];
+      conv.entry_of = iptr(6);
+    }
     ops.diff_qk_prep(arg(0), fptr(1), fptr(2), (float)num(0), r, iptr(5), iptr(6), view_of(7, arg(8)), arg(8), arg(9), (int)num(1),
-                     (int)num(2), (int)num(3), (int)num(4));
+                     (int)num(2), (int)num(3), (int)num(4), with_conv ? &conv : nullptr);
   } else if (op == "diff_attention") {
     // q, pool, table, positions, slots, out, [tiles [n, 3], rows [n], entries [R, 4]]; heads, kv_heads, dk, dv, scale, block,
     // window, lambda, eps, out_scale, [rows of single tokens where no list names them]

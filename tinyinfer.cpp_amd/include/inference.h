@@ -351,8 +351,9 @@ class Ops {
   // ---- layers that norm what a sublayer returns; short convolutions; differential attention; mixtures of experts
   // x (+)= y / rms(y) * gain (32-bit; gain is the factor itself).  accumulate false: x is overwritten (y may be x).
   // gather (device int32 [M][n_gather]): row m of y is the sum of the rows y[gather[m][k]], k ascending
+  // rounded (may be null): also receives the new x in its own dtype, for the product that reads the residual next
   void norm_residual(const Tensor& x, const Tensor& y, const Tensor& gain, float eps, bool accumulate, const int* gather = nullptr,
-                     int n_gather = 0);
+                     int n_gather = 0, const Tensor* rounded = nullptr);
   void round_rows(const Tensor& x, const Tensor& out);                               // out = x in out's dtype
   void scale(const Tensor& x, float s);                                              // x *= s (float32)
   // out[m, c] = sum_j taps[c, j] u(position of m - (K - 1) + j)[c] over each entry's rows, the K - 1 rows before an
@@ -361,9 +362,11 @@ class Ops {
                   const int* entry_of, const int* positions, const Tensor& out);
   // qkv f32 [M, heads 2 dk + kv_heads 2 dk + kv_heads dv] (two maps a head): per-map norm, rotation of the first
   // rot.dims entries, q to q_out, k and v into pages K [kv][P][2 dk] | V [kv][dv][P]
+  // conv (may be null): the short convolution of `short_conv` on every channel first, inside the same kernel
+  struct ShortConv { Tensor taps, state; const int* entry_meta = nullptr; int n_entries = 0; const int* entry_of = nullptr; };
   void diff_qk_prep(const Tensor& qkv, const float* q_w, const float* k_w, float eps, const Rotation& rot, const int* positions,
                     const int* slots, const CacheView& view, const Tensor& pool, const Tensor& q_out, int heads, int kv_heads,
-                    int dk, int dv);
+                    int dk, int dv, const ShortConv* conv = nullptr);
   // differential attention of every row over such pages: (a1 - lambda a2) / rms * out_scale per head; a key is visible
   // inside the query's block of `block` positions (0: no blocks) and window (0: none)
   // lists (device int32, the step's metadata): tiles [n_tiles][3] = (entry, first row, rows <= 64) of the entries of several
@@ -606,8 +609,9 @@ class NormPart : public Part { public: using Part::Part; const char* family() co
   // x (+)= norm(y), both f32 [M, dim], in 32-bit: for arrangements that norm what a sublayer returns (y may be x itself
   // when nothing is accumulated)
   virtual bool can_add() const { return false; }
+  // rounded (may be null): also receives the new x in its own dtype
   virtual void forward_add(StepContext& ctx, const Tensor& y, const Tensor& x, bool accumulate, const int* gather = nullptr,
-                           int n_gather = 0); };
+                           int n_gather = 0, const Tensor* rounded = nullptr); };
 class PositionPart : public Part { public: using Part::Part; const char* family() const override { return "pos"; }
   virtual bool fused(Ops::Rotation& rot) const { return false; }    // arguments for the fused q/k kernels
   virtual bool additive() const { return false; }                   // an encoding added to the residual behind the embedding ...
@@ -621,7 +625,9 @@ class MixerPart : public Part { public: using Part::Part; const char* family() c
   virtual bool takes_lazy_norm() const { return false; } };        // h goes into exactly one Ops::linear
 // an operation along time on every channel of the step's rows, with what it must remember of a request as its state
 class FilterPart : public Part { public: using Part::Part; const char* family() const override { return "filter"; }
-  virtual void forward(StepContext& ctx, const Tensor& u, const Tensor& out) = 0; };
+  virtual void forward(StepContext& ctx, const Tensor& u, const Tensor& out) = 0;
+  // a short convolution that the kernel behind it can take in: its taps and state for this step (false: run forward)
+  virtual bool fused(StepContext& ctx, Ops::ShortConv& conv) { return false; } };
 class FeedForwardPart : public Part { public: using Part::Part; const char* family() const override { return "ffn"; }
   virtual void forward(StepContext& ctx, const Rows& h, const Tensor& x) = 0;
   virtual bool can_store() const { return false; }

@@ -355,9 +355,10 @@ class Ops:
         self._call("gated_head_norm", [o, proj, w, out], [gate_col, eps, heads, dv])
 
     # ---- post-norm layers, short convolutions, differential attention, mixtures of experts
-    def norm_residual(self, x, y, gain, eps, accumulate=True, gather=None):
-        """x (+)= y / rms(y) * gain, all float32; gather int32 [M, n]: row m of y is the sum of the rows y[gather[m, k]]."""
-        self._call("norm_residual", [x, y, gain, gather], [eps, int(bool(accumulate))])
+    def norm_residual(self, x, y, gain, eps, accumulate=True, gather=None, rounded=None):
+        """x (+)= y / rms(y) * gain, all float32; gather int32 [M, n]: row m of y is the sum of the rows y[gather[m, k]];
+        rounded: also receives the new x in its own dtype."""
+        self._call("norm_residual", [x, y, gain, gather, rounded], [eps, int(bool(accumulate))])
 
     def round_rows(self, x, out):
         self._call("round_rows", [x, out])
@@ -371,10 +372,14 @@ class Ops:
         self._call("short_conv", [u, taps, state, entries, entry_of, positions, out])
 
     def diff_qk_prep(self, qkv, q_w, k_w, inv_freq, rope_table, positions, slots, table, pool, q_out, eps, heads, kv_heads, dk, dv,
-                     rot_dims=0, mag=1.0):
-        """qkv f32 [M, heads 2 dk + kv_heads (2 dk + dv)]; pool [pages, kv_heads, P, 2 dk + dv] (K [kv][P][2 dk] | V [kv][dv][P])."""
-        self._call("diff_qk_prep", [qkv, q_w, k_w, inv_freq, rope_table, positions, slots, table, pool, q_out],
-                   [eps, heads, kv_heads, dk, dv, rot_dims, mag])
+                     rot_dims=0, mag=1.0, taps=None, state=None, entries=None):
+        """qkv f32 [M, heads 2 dk + kv_heads (2 dk + dv)]; pool [pages, kv_heads, P, 2 dk + dv] (K [kv][P][2 dk] | V [kv][dv][P]).
+        taps f32 [C, K] with state f32 [slots, K - 1, C] and entries int32 [R, 4] (slots names every row's entry): the short
+        convolution of `short_conv` on every channel first, inside the same kernel."""
+        tensors = [qkv, q_w, k_w, inv_freq, rope_table, positions, slots, table, pool, q_out]
+        if taps is not None:
+            tensors += [taps, state, entries]
+        self._call("diff_qk_prep", tensors, [eps, heads, kv_heads, dk, dv, rot_dims, mag])
 
     def diff_attention(self, q, pool, table, positions, slots, out, heads, kv_heads, dk, dv, scale, lam, eps, out_scale, block=0, window=0,
                        tiles=None, rows=None, entries=None, all_rows=False):

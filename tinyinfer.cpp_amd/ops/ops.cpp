@@ -995,14 +995,16 @@ void Ops::gated_head_norm(const Tensor& o, const Tensor& proj, int gate_col, con
 
 // ------------------------------------------------- post-norm layers, short convolutions, differential attention, experts
 void Ops::norm_residual(const Tensor& x, const Tensor& y, const Tensor& gain, float eps, bool accumulate, const int* gather,
-                        int n_gather) {
+                        int n_gather, const Tensor* rounded) {
   TIMED("norm_residual " + dims(x));
   const int64_t H = x.ndim == 2 ? x.shape[1] : 0;
   require(x.ndim == 2 && x.dtype == DType::F32 && x.contiguous() && y.ndim == 2 && y.dtype == DType::F32 && y.contiguous() &&
               y.shape[1] == H && (gather ? n_gather > 0 : y.shape[0] == x.shape[0]) && gain.dtype == DType::F32 && gain.numel() == H,
           "norm_residual: x " + x.describe() + ", y " + y.describe() + " or gain " + gain.describe() + " do not fit");
+  require(!rounded || (rounded->contiguous() && rounded->numel() == x.numel()), "norm_residual: the rounded copy does not fit x");
   int rc = KERNEL("residual", ti_norm_residual)((float*)x.data, (const float*)y.data, (const float*)gain.data, gather, n_gather,
-                                                (int)x.shape[0], (int)H, eps, accumulate ? 1 : 0, (hipStream_t)launch_stream());
+                                                (int)x.shape[0], (int)H, eps, accumulate ? 1 : 0, rounded ? rounded->data : nullptr,
+                                                rounded ? code(rounded->dtype, "norm_residual") : 0, (hipStream_t)launch_stream());
   check("residual", rc, "norm_residual");
 }
 
@@ -1044,8 +1046,8 @@ void Ops::short_conv(const Tensor& u, const Tensor& taps, const Tensor& state, c
 
 void Ops::diff_qk_prep(const Tensor& qkv, const float* q_w, const float* k_w, float eps, const Rotation& rot, const int* positions,
                        const int* slots, const CacheView& view, const Tensor& pool, const Tensor& q_out, int heads, int kv_heads,
-                       int dk, int dv) {
-  TIMED("diff_qk_prep " + dims(qkv));
+                       int dk, int dv, const ShortConv* conv) {
+  TIMED("diff_qk_prep " + dims(qkv) + (conv ? " conv" : ""));
   const int64_t M = qkv.shape[0];
   const int64_t width = (int64_t)heads * 2 * dk + (int64_t)kv_heads * (2 * dk + dv);
   require(qkv.ndim == 2 && qkv.shape[1] == width && qkv.dtype == DType::F32 && qkv.contiguous(),
@@ -1054,7 +1056,21 @@ void Ops::diff_qk_prep(const Tensor& qkv, const float* q_w, const float* k_w, fl
           "diff_qk_prep: q_out has the wrong shape");
   check_split_pool("diff_qk_prep", pool, kv_heads, 2 * dk, dv, q_out.dtype);
   const int rot_dims = rot.inv_freq ? (rot.dims > 0 ? rot.dims : dk) : 0;
-  int rc = KERNEL("diff_attention", ti_diff_qk_prep)(code(q_out.dtype, "diff_qk_prep"), (const float*)qkv.data, q_w, k_w, eps,
+  int K = 0;
+  if (conv) {
+    require(conv->taps.ndim == 2 && conv->taps.dtype == DType::F32 && conv->taps.contiguous() && conv->taps.shape[0] == width,
+            "diff_qk_prep: taps " + conv->taps.describe() + " must be float32 [" + std::to_string(width) + ", taps]");
+    K = (int)conv->taps.shape[1];
+    require(K == 1 || (conv->state.defined() && conv->state.dtype == DType::F32 && conv->state.contiguous() && conv->state.ndim == 3 &&
+                       conv->state.shape[1] == K - 1 && conv->state.shape[2] == width),
+            "diff_qk_prep: the convolution's state " + conv->state.describe() + " does not fit");
+    require(conv->entry_meta && conv->entry_of, "diff_qk_prep: the convolution needs the entry records");
+    took("[fused]");
+  }
+  int rc = KERNEL("diff_attention", ti_diff_qk_prep)(code(q_out.dtype, "diff_qk_prep"), (const float*)qkv.data,
+                                                     conv ? (const float*)conv->taps.data : nullptr,
+                                                     conv ? (float*)conv->state.data : nullptr, conv ? conv->entry_meta : nullptr,
+                                                     conv ? conv->n_entries : 0, conv ? conv->entry_of : nullptr, K, q_w, k_w, eps,
                                                      rot.inv_freq, rot.table, rot.table_len, rot.mag, rot_dims, positions, slots,
                                                      view.table, view.table_width, pool.data, q_out.data, (int)M, heads, kv_heads, dk,
                                                      dv, (int)pool.shape[2], (hipStream_t)launch_stream());

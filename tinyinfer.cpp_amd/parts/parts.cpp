@@ -101,7 +101,7 @@ std::string tensor_name(const Json& p, const char* key, const std::string& prefi
 }
 }  // namespace
 
-void NormPart::forward_add(StepContext&, const Tensor&, const Tensor&, bool, const int*, int) {
+void NormPart::forward_add(StepContext&, const Tensor&, const Tensor&, bool, const int*, int, const Tensor*) {
   throw EngineError(std::string("the norm '") + kind_name() + "' cannot write into the residual");
 }
 void MixerPart::forward_store(StepContext&, const Rows&, const Tensor&) {
@@ -305,8 +305,9 @@ class RMSNorm final : public NormPart {
   static void spread(const Tensor& one, const Tensor& all, bool on_host);     // all[:] = one[0]
   static void plus_one(const Tensor& w, const Tensor& out, bool on_host);     // out = 1 + w
   bool can_add() const override { return true; }
-  void forward_add(StepContext& ctx, const Tensor& y, const Tensor& x, bool accumulate, const int* gather, int n_gather) override {
-    ctx.ops.norm_residual(x, y, weight, eps, accumulate, gather, n_gather);
+  void forward_add(StepContext& ctx, const Tensor& y, const Tensor& x, bool accumulate, const int* gather, int n_gather,
+                   const Tensor* rounded) override {
+    ctx.ops.norm_residual(x, y, weight, eps, accumulate, gather, n_gather, rounded);
   }
   // x: f32 [M, dim].  With `rows` only those rows of x are read, in that order.  `lazy`: the
   // consumer feeds the result to one product and nothing else, so where a kernel can take the
@@ -1256,13 +1257,21 @@ class ShortConv final : public FilterPart {
     n.state_shape = {(int64_t)taps - 1, channels};
     return n;
   }
+  Tensor state_of(StepContext& ctx) const {
+    if (taps == 1) return Tensor();
+    const auto bound = ctx.binding(this);
+    return ctx.state(bound.first, bound.second);
+  }
   void forward(StepContext& ctx, const Tensor& u, const Tensor& out) override {
-    Tensor state;
-    if (taps > 1) {
-      const auto bound = ctx.binding(this);
-      state = ctx.state(bound.first, bound.second);
-    }
-    ctx.ops.short_conv(u, w, state, ctx.entry_meta, (int)ctx.entries.size(), ctx.slots, ctx.positions, out);
+    ctx.ops.short_conv(u, w, state_of(ctx), ctx.entry_meta, (int)ctx.entries.size(), ctx.slots, ctx.positions, out);
+  }
+  bool fused(StepContext& ctx, Ops::ShortConv& conv) override {
+    conv.taps = w;
+    conv.state = state_of(ctx);
+    conv.entry_meta = ctx.entry_meta;
+    conv.n_entries = (int)ctx.entries.size();
+    conv.entry_of = ctx.slots;
+    return true;
   }
   std::vector<std::pair<std::string, Tensor>> held() const override { return {{"w", w}}; }
   int taps = 1;
@@ -1437,7 +1446,10 @@ class DiffAttention final : public MixerPart {
     const int64_t width = nq + nk + nv;
     Tensor qkv = ctx.buf("dattn.qkv", DType::F32, {M, width});
     ctx.ops.linear(h, w_qkv, qkv, Ops::Store);
-    if (conv) {
+    // the convolution inside the kernel that prepares queries and keys, where the filter has a form for that
+    Ops::ShortConv taken;
+    const bool conv_inside = conv && conv->fused(ctx, taken);
+    if (conv && !conv_inside) {
       Tensor mixed = ctx.buf("dattn.conv", DType::F32, {M, width});
       conv->forward(ctx, qkv, mixed);
       qkv = mixed;
@@ -1449,7 +1461,7 @@ class DiffAttention final : public MixerPart {
     if (pos && !pos->fused(rot)) throw EngineError("diff_attention: the position encoding '" + std::string(pos->kind_name()) + "' has no fused form");
     Tensor q = ctx.buf("dattn.q", ctx.act_dtype, {M, nq});
     ctx.ops.diff_qk_prep(qkv, q_norm_w.ptr<float>(), k_norm_w.ptr<float>(), eps, rot, ctx.positions, ctx.slots, view, pool, q, heads,
-                         kv_heads, dk, dv);
+                         kv_heads, dk, dv, conv_inside ? &taken : nullptr);
     Tensor a = ctx.buf("dattn.out", ctx.act_dtype, {M, no});
     const Ops::DiffAttentionLists l = lists(ctx);
     ctx.ops.diff_attention(q, pool, view, ctx.positions, ctx.slots, a, heads, kv_heads, dk, dv, scale, block, window, lambda, eps,
@@ -1610,10 +1622,21 @@ class PostNormBlock final : public BlockPart {
   void forward(StepContext& ctx, const Tensor& x) override {
     Tensor y = ctx.buf("post_norm.y", DType::F32, {x.shape[0], x.shape[1]});
     mixer->forward_store(ctx, input(ctx, x), y);
-    norm1->forward_add(ctx, y, x, true);
-    if (!ffn) return;
+    if (!ffn) {
+      norm1->forward_add(ctx, y, x, true);
+      return;
+    }
+    // the kernel that adds the normed rows also leaves the rounding of the new residual for the feed-forward
+    Rows h;
+    if (ctx.act_dtype == DType::F32) {
+      norm1->forward_add(ctx, y, x, true);
+      h.t = x;
+    } else {
+      h.t = ctx.buf("post_norm.h", ctx.act_dtype, {x.shape[0], x.shape[1]});
+      norm1->forward_add(ctx, y, x, true, nullptr, 0, &h.t);
+    }
     Ops::GatheredRows rows;
-    ffn->forward_rows(ctx, input(ctx, x), y, rows);
+    ffn->forward_rows(ctx, h, y, rows);
     norm2->forward_add(ctx, rows.t, x, true, rows.gather, rows.n_gather);
   }
   std::shared_ptr<NormPart> norm1, norm2;
