@@ -253,12 +253,15 @@ def test_prepared_keys_and_differential_attention(ops, dtype, heads, kv, dk, dv,
         args = (q_out, pool, dev(table, torch.int32), dev(pos, torch.int32), dev(slots, torch.int32))
         calls = ops.timing_report() and None
         ops.count_calls(True)
-        for lists in (dict(tiles=tiles, entries=entries), dict(all_rows=True),
-                      dict(tiles=tiles[:1], entries=entries, rows=dev(list(range(64, T)), torch.int32))):
-            fast = torch.zeros(T, heads * dv, device="cuda", dtype=DT[dtype])
-            ops.diff_attention(*args, fast, heads, kv, dk, dv, scale, lam, eps, out_scale, block=block, **lists)
-            err = np.abs(f64(fast) - want)
-            assert err.max() < bound, (list(lists), np.unravel_index(err.argmax(), err.shape), err.max())
+        for shared in (True, False):       # a tile's wavefronts share keys and values through LDS, or each fetches its own
+            ops.use_shared_tiles = shared
+            for lists in (dict(tiles=tiles, entries=entries), dict(all_rows=True),
+                          dict(tiles=tiles[:1], entries=entries, rows=dev(list(range(64, T)), torch.int32))):
+                fast = torch.zeros(T, heads * dv, device="cuda", dtype=DT[dtype])
+                ops.diff_attention(*args, fast, heads, kv, dk, dv, scale, lam, eps, out_scale, block=block, **lists)
+                err = np.abs(f64(fast) - want)
+                assert err.max() < bound, (shared, list(lists), np.unravel_index(err.argmax(), err.shape), err.max())
+        ops.use_shared_tiles = True
         took = [c["name"] for c in ops.timing_report()]
         ops.count_calls(False)
         assert took and all("[mfma]" in n for n in took), took

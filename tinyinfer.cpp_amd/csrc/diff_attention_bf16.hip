@@ -278,6 +278,174 @@ diff_tiles_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool,
   finish_column<DV>(st, lambda, eps, out_scale, out + ((size_t)row * n_head + h) * DV, live);
 }
 
+// ------------------------------------------------------------------------------------------ tiles, keys and values through LDS
+// The same tiles with the four wavefronts sharing what they read: a pair of blocks (32 keys: their two maps and the values)
+// is fetched once by the workgroup into one of two LDS stages while the pair before it is multiplied from the other, one
+// barrier a pair.  Key rows are padded by 16 bytes and value rows by 8, so that the fragments' reads spread over the banks.
+template <int DK, int DV>
+struct DiffStage {
+  static constexpr int KROW = 2 * DK + 8;       // bfloat16 elements of a key row
+  static constexpr int VROW = 32 + 4;           // of a value row: 32 keys (block A, block B)
+  static constexpr int K_ELEMS = 32 * KROW, ELEMS = K_ELEMS + DV * VROW;
+  static constexpr int K_UNITS = 32 * (2 * DK / 8), V_UNITS = DV * 4;      // 16-byte pieces fetched per pair
+  static constexpr int K_PER = (K_UNITS + 255) / 256, V_PER = (V_UNITS + 255) / 256;
+};
+
+// the workgroup's fetch of a pair into registers (thread t the 16-byte pieces t, t + 256, ...), and their way into a stage
+template <int DK, int DV>
+__device__ __forceinline__ void fetch_pair(const bf16_t* ka, const bf16_t* kb, const bf16_t* va, const bf16_t* vb, int P,
+                                           uint4 (&kreg)[DiffStage<DK, DV>::K_PER], uint4 (&vreg)[DiffStage<DK, DV>::V_PER]) {
+  using S = DiffStage<DK, DV>;
+#pragma unroll
+  for (int i = 0; i < S::K_PER; ++i) {
+    const int u = threadIdx.x + 256 * i;
+    if (S::K_UNITS % 256 == 0 || u < S::K_UNITS) {
+      const int key = u / (2 * DK / 8), part = u % (2 * DK / 8);
+      kreg[i] = *reinterpret_cast<const uint4*>((key < 16 ? ka : kb) + (size_t)(key & 15) * (2 * DK) + part * 8);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < S::V_PER; ++i) {
+    const int u = threadIdx.x + 256 * i;
+    if (S::V_UNITS % 256 == 0 || u < S::V_UNITS) {
+      const int d = u >> 2, piece = u & 3;
+      vreg[i] = *reinterpret_cast<const uint4*>(((piece & 2) ? vb : va) + (size_t)d * P + (piece & 1) * 8);
+    }
+  }
+}
+template <int DK, int DV>
+__device__ __forceinline__ void park_pair(bf16_t* to, const uint4 (&kreg)[DiffStage<DK, DV>::K_PER],
+                                          const uint4 (&vreg)[DiffStage<DK, DV>::V_PER]) {
+  using S = DiffStage<DK, DV>;
+#pragma unroll
+  for (int i = 0; i < S::K_PER; ++i) {
+    const int u = threadIdx.x + 256 * i;
+    if (S::K_UNITS % 256 == 0 || u < S::K_UNITS) {
+      const int key = u / (2 * DK / 8), part = u % (2 * DK / 8);
+      *reinterpret_cast<uint4*>(to + key * S::KROW + part * 8) = kreg[i];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < S::V_PER; ++i) {
+    const int u = threadIdx.x + 256 * i;
+    if (S::V_UNITS % 256 == 0 || u < S::V_UNITS) {
+      const int d = u >> 2, piece = u & 3;
+      uint2* dst = reinterpret_cast<uint2*>(to + S::K_ELEMS + d * S::VROW + (piece >> 1) * 16 + (piece & 1) * 8);
+      dst[0] = make_uint2(vreg[i].x, vreg[i].y);
+      dst[1] = make_uint2(vreg[i].z, vreg[i].w);
+    }
+  }
+}
+
+template <int DK, int DV>
+__global__ void __launch_bounds__(256)
+diff_tiles_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool, const int* __restrict__ table, int table_stride,
+                      const int* __restrict__ tiles, const int* __restrict__ entries, bf16_t* __restrict__ out, int n_head, int n_kv,
+                      int P, float scale2, int block, int window, float lambda, float eps, float out_scale) {
+  using S = DiffStage<DK, DV>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  bf16_t* const lds = reinterpret_cast<bf16_t*>(lds_raw);      // two stages of S::ELEMS
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r16 = lane & 15, quad = lane >> 4;
+  const int e = tiles[3 * blockIdx.x], tile_row0 = tiles[3 * blockIdx.x + 1], tile_rows = tiles[3 * blockIdx.x + 2];
+  const int row0 = tile_row0 + 16 * wave, n_rows = tile_rows - 16 * wave;      // n_rows <= 0: a wavefront without rows (it still fetches)
+  const int h = blockIdx.y;
+  const int kvh = h / (n_head / n_kv);
+  const int e_row0 = entries[4 * e], e_n = entries[4 * e + 1], e_start = entries[4 * e + 2];
+  const int kv_last = e_start + e_n - 1;
+  const bool live = r16 < n_rows;
+  const int row = live ? row0 + r16 : tile_row0;
+  const int p = e_start + (row - e_row0);
+  const int lo = live ? first_visible(p, block, window) : 1, hi = live ? p : 0;
+  int lo_min = live ? lo : 0x7fffffff, lo_max = live ? lo : 0, hi_min = live ? hi : 0x7fffffff, hi_max = live ? hi : -1;
+#pragma unroll
+  for (int o = 1; o < 16; o <<= 1) {
+    lo_min = min(lo_min, __shfl_xor(lo_min, o, 64));
+    lo_max = max(lo_max, __shfl_xor(lo_max, o, 64));
+    hi_min = min(hi_min, __shfl_xor(hi_min, o, 64));
+    hi_max = max(hi_max, __shfl_xor(hi_max, o, 64));
+  }
+  // the workgroup's range of pairs: from the first key its first row sees to its last row's own
+  const int p_first = e_start + (tile_row0 - e_row0), p_last = p_first + tile_rows - 1;
+  const int pair0 = first_visible(p_first, block, window) / 32, pair1 = p_last / 32 + 1;
+  const int* tab = table + (size_t)e * table_stride;
+  const size_t page_elems = (size_t)n_kv * P * (2 * DK + DV);
+  const size_t v_base = (size_t)n_kv * P * (2 * DK) + (size_t)kvh * DV * P;
+
+  Frag8 qf[2][DK / 32];
+  const bf16_t* qrow = q + ((size_t)row * n_head + h) * 2 * DK + quad * 8;
+#pragma unroll
+  for (int mp = 0; mp < 2; ++mp)
+#pragma unroll
+    for (int s = 0; s < DK / 32; ++s) qf[mp][s].u = *reinterpret_cast<const uint4*>(qrow + mp * DK + s * 32);
+  MapState<DV> st[2];
+  st[0].clear();
+  st[1].clear();
+
+  uint4 kreg[S::K_PER], vreg[S::V_PER];
+  bool validA = false, validB = false;      // of the pair in flight; the same in every lane
+  auto fetch = [&](int pair) __attribute__((always_inline)) {
+    const int keyA = pair * 32, keyB = keyA + 16;
+    int pageA = keyA <= kv_last ? tab[keyA / P] : -1;
+    int pageB = keyB <= kv_last ? tab[keyB / P] : -1;
+    validA = pageA >= 0;
+    validB = pageB >= 0;
+    int rowA = keyA % P, rowB = keyB % P;
+    if (pageA < 0) {
+      pageA = tab[p_last / P];
+      rowA = p_last / 16 * 16 % P;
+    }
+    if (pageB < 0) {
+      pageB = tab[p_last / P];
+      rowB = p_last / 16 * 16 % P;
+    }
+    const bf16_t* ka = pool + (size_t)pageA * page_elems + ((size_t)kvh * P + rowA) * (2 * DK);
+    const bf16_t* kb = pool + (size_t)pageB * page_elems + ((size_t)kvh * P + rowB) * (2 * DK);
+    fetch_pair<DK, DV>(ka, kb, pool + (size_t)pageA * page_elems + v_base + rowA, pool + (size_t)pageB * page_elems + v_base + rowB, P,
+                       kreg, vreg);
+  };
+  auto park = [&](bf16_t* to) __attribute__((always_inline)) { park_pair<DK, DV>(to, kreg, vreg); };
+
+  fetch(pair0);
+  park(lds);
+  bool curA = validA, curB = validB;
+  __syncthreads();
+  for (int pair = pair0, cur = 0; pair < pair1; ++pair, cur ^= 1) {
+    const bool more = pair + 1 < pair1;
+    if (more) fetch(pair + 1);
+    const int keyA = pair * 32;
+    if (n_rows > 0 && keyA <= hi_max && keyA + 31 >= lo_min) {
+      DiffPair<DK, DV> f;
+      f.keyA = keyA;
+      f.keyB = keyA + 16;
+      f.validA = curA;
+      f.validB = curB;
+      const bf16_t* ks = lds + cur * S::ELEMS;
+      const bf16_t* vs = ks + S::K_ELEMS;
+#pragma unroll
+      for (int mp = 0; mp < 2; ++mp)
+#pragma unroll
+        for (int s = 0; s < DK / 32; ++s) {
+          f.k[0][mp][s].u = *reinterpret_cast<const uint4*>(ks + r16 * S::KROW + mp * DK + s * 32 + quad * 8);
+          f.k[1][mp][s].u = *reinterpret_cast<const uint4*>(ks + (16 + r16) * S::KROW + mp * DK + s * 32 + quad * 8);
+        }
+#pragma unroll
+      for (int d = 0; d < DV / 16; ++d) {
+        const bf16_t* vr = vs + (16 * d + r16) * S::VROW + quad * 4;
+        const uint2 a = *reinterpret_cast<const uint2*>(vr), b = *reinterpret_cast<const uint2*>(vr + 16);
+        f.v[d].u = make_uint4(a.x, a.y, b.x, b.y);
+      }
+      const bool plain = curA && curB && keyA >= lo_max && keyA + 31 <= hi_min;
+      attend_pair<DK, DV>(f, qf, lo, hi, plain, kv_last, scale2, st);
+    }
+    if (more) park(lds + (cur ^ 1) * S::ELEMS);
+    curA = validA;
+    curB = validB;
+    __syncthreads();
+  }
+  if (n_rows > 0) finish_column<DV>(st, lambda, eps, out_scale, out + ((size_t)row * n_head + h) * DV, live);
+}
+
 // ------------------------------------------------------------------------------------------ single rows
 // rows int32 [n] (null: row r is r); the 16 columns are the query heads of kv head blockIdx.y.  The four wavefronts take
 // the pairs of blocks in turns; wavefronts 1..3 leave their state in LDS and the first one merges and finishes.
@@ -366,7 +534,7 @@ static bool served(int dk, int dv, int page_size, int n_head, int n_kv) {
 extern "C" int ti_diff_attention_tiles_bf16(const void* q, const void* pool, const int* table, int table_stride, const int* tiles,
                                             const int* entries, void* out, int n_tiles, int n_head, int n_kv, int dk, int dv,
                                             int page_size, float scale, int block, int window, float lambda, float eps,
-                                            float out_scale, hipStream_t stream) {
+                                            float out_scale, int use_lds, hipStream_t stream) {
   if (!served(dk, dv, page_size, n_head, n_kv)) {
     ti_set_error("diff_attention (tiles): sizes %d / %d, pages of %d are not served", dk, dv, page_size);
     return 3;
@@ -374,10 +542,18 @@ extern "C" int ti_diff_attention_tiles_bf16(const void* q, const void* pool, con
   TI_REQUIRE(n_head <= 65535 && table_stride > 0 && block >= 0 && window >= 0, "diff_attention (tiles): bad arguments");
   if (n_tiles == 0) return 0;
   dim3 grid(n_tiles, n_head);
-#define DA_TILES(K, V)                                                                                                           \
-  diff_tiles_kernel<K, V><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, entries, \
-                                                    (bf16_t*)out, n_head, n_kv, page_size, scale * DA_LOG2E, block, window,      \
-                                                    lambda, eps, out_scale)
+  // keys and values shared through LDS (use_lds 0: every wavefront fetches its own, for tests and measurements)
+#define DA_TILES(K, V)                                                                                                              \
+  do {                                                                                                                              \
+    if (use_lds)                                                                                                                    \
+      diff_tiles_lds_kernel<K, V><<<grid, 256, 2 * DiffStage<K, V>::ELEMS * 2, stream>>>(                                           \
+          (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, entries, (bf16_t*)out, n_head, n_kv, page_size,        \
+          scale * DA_LOG2E, block, window, lambda, eps, out_scale);                                                                 \
+    else                                                                                                                            \
+      diff_tiles_kernel<K, V><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, entries, \
+                                                        (bf16_t*)out, n_head, n_kv, page_size, scale * DA_LOG2E, block, window,     \
+                                                        lambda, eps, out_scale);                                                    \
+  } while (0)
   DA_DISPATCH(DA_TILES);
 #undef DA_TILES
   TI_LAUNCH_CHECK();

@@ -172,7 +172,8 @@ int ti_diff_attention_rows(int dtype, const void* q, const void* pool, const int
 int ti_diff_attention_tiles_bf16(const void* q, const void* pool, const int* table, int table_stride, const int* tiles,
                                  const int* entries, void* out, int n_tiles, int n_head, int n_kv, int dk, int dv,
                                  int page_size, float scale, int block, int window, float lambda, float eps, float out_scale,
-                                 hipStream_t stream);
+                                 int use_lds, hipStream_t stream);
+// (use_lds 1: the four wavefronts of a tile share the keys and values they read through LDS; 0: each fetches its own)
 // single rows (rows int32 [n_rows], or null: rows 0 .. n_rows - 1); at most 16 query heads a kv head
 int ti_diff_attention_rows_bf16(const void* q, const void* pool, const int* table, int table_stride, const int* pos,
                                 const int* slot, const int* rows, void* out, int n_rows, int n_head, int n_kv, int dk, int dv,

@@ -414,6 +414,7 @@ class Ops {
     bool split_k_add = true, deferred_add = true, paired_prefill = true, portion_splits = true;
     bool early_page_ids = true;     // a step of single tokens: the decode attention fetches a row's page ids beside its position
     bool radix_sample = true;       // draws with a top-k cut: many workgroups share a row (else one walks it bit by bit)
+    bool shared_tiles = true;       // differential attention over a portion: a tile's wavefronts share keys and values through LDS
     int force_paired_tiles = -1;    // 1 / 0: that kernel with / without pairs, whatever the launch
     int force_decode_splits = 0;    // > 0: the decode attention cuts every context into this many runs
   } use;

@@ -1094,7 +1094,7 @@ void Ops::diff_attention(const Tensor& q, const Tensor& pool, const CacheView& v
       rc = KERNEL("diff_attention_bf16", ti_diff_attention_tiles_bf16)(q.data, pool.data, view.table, view.table_width, lists->tiles,
                                                                        lists->entry_meta, out.data, lists->n_tiles, heads, kv_heads, dk,
                                                                        dv, (int)pool.shape[2], scale, block, window, lambda, eps,
-                                                                       out_scale, (hipStream_t)launch_stream());
+                                                                       out_scale, use.shared_tiles ? 1 : 0, (hipStream_t)launch_stream());
     if (rc == 0 && lists->n_rows)
       rc = KERNEL("diff_attention_bf16", ti_diff_attention_rows_bf16)(q.data, pool.data, view.table, view.table_width, positions, slots,
                                                                       lists->rows, out.data, lists->n_rows, heads, kv_heads, dk, dv,

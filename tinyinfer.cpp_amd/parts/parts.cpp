@@ -1414,7 +1414,10 @@ class DiffAttention final : public MixerPart {
     }
     int* tiles = plan.ints("dattn.tiles", 3 * n_tiles);
     int* rows = plan.ints("dattn.rows", n_rows);
-    size_t t = 0, r = 0;
+    struct Tile { int keys, entry, row, n; };
+    std::vector<Tile> order;
+    order.reserve(n_tiles);
+    size_t r = 0;
     for (size_t i = 0; i < entries.size(); ++i) {
       const auto& e = entries[i];
       if (e.n_tokens == 1) {
@@ -1422,10 +1425,17 @@ class DiffAttention final : public MixerPart {
         continue;
       }
       for (int q0 = 0; q0 < e.n_tokens; q0 += TILE_ROWS) {
-        tiles[t++] = (int)i;
-        tiles[t++] = e.row0 + q0;
-        tiles[t++] = std::min(TILE_ROWS, e.n_tokens - q0);
+        const int n = std::min(TILE_ROWS, e.n_tokens - q0);
+        const int last = e.start + q0 + n - 1;                       // the tile's last position, and how many keys it sees
+        order.push_back({block > 0 ? last % block + 1 : last + 1, (int)i, e.row0 + q0, n});
       }
+    }
+    // from the tile that walks the most keys to the one that walks the fewest: the long ones start first
+    std::stable_sort(order.begin(), order.end(), [](const Tile& a, const Tile& b) { return a.keys > b.keys; });
+    for (size_t t = 0; t < order.size(); ++t) {
+      tiles[3 * t] = order[t].entry;
+      tiles[3 * t + 1] = order[t].row;
+      tiles[3 * t + 2] = order[t].n;
     }
   }
   Ops::DiffAttentionLists lists(const StepContext& ctx) const {
