@@ -1,12 +1,12 @@
 // The experts of a mixture of experts for steps of many tokens, bfloat16 on the matrix cores of gfx950.
 //
 //   1. moe_group: counts the (token, expert) pairs of every expert, lays the experts' runs of rows one after
-//      the other and cuts them into tiles of 64 rows: offsets, the list of tiles, cursors at zero.
+//      the other and cuts them into tiles of 128 rows: offsets, the list of tiles, cursors at zero.
 //   2. moe_place: every pair takes the next free row of its expert's run (which row does not matter: a row of
 //      a product depends on no other row) and writes its scaled input there, rounded to bfloat16.
 //   3. two grouped products over the tiles: act = relu(A up_e^T)^2 (bfloat16), out = act down_e^T (32-bit).
-//      Weights are the A operand of v_mfma_f32_16x16x32_bf16 and tokens the 16 columns, both straight from
-//      memory in their own layouts; a lane ends with four consecutive outputs of one token.
+//      Weights are the A operand of v_mfma_f32_16x16x32_bf16 and tokens the 16 columns, both in their own
+//      layouts through LDS; a lane ends with four consecutive outputs of one token.
 //   4. a token's rows are added in the order its experts were chosen: by the norm that reads them next
 //      (it is handed the list `where`), or by moe_combine.
 #include "common.h"
@@ -21,7 +21,7 @@ union Frag8 {
   bf16x8 v;
 };
 
-#define MOE_TILE 64          // rows (pairs) of a tile
+#define MOE_TILE 128         // rows (pairs) of a tile
 #define MOE_MAX_E 1024
 
 // meta int32: [0] number of tiles, [1 .. E + 1] offsets of the experts' runs, then E cursors, then tiles [max][3] =
@@ -87,58 +87,75 @@ moe_place_kernel(const bf16_t* __restrict__ h, const int* __restrict__ ids, cons
   }
 }
 
-// out[row][n] (op)= sum_k rows[row][k] w[e][n][k] over the tiles.  A workgroup: one tile of 64 rows x 256 outputs; wavefront v
-// the outputs 64 v .. 64 v + 63 of it (four blocks of 16) against the four blocks of 16 rows: sixteen matrix instructions for
-// eight 16-byte loads a lane.  EPI 0: relu^2, bfloat16; 1: 32-bit.
+// out[row][n] (op)= sum_k rows[row][k] w[e][n][k] over the tiles.  A workgroup: one tile of 128 rows x 128 outputs, its four
+// wavefronts two by two, each 64 outputs (four blocks of 16) against 64 rows (four blocks of 16).  A step of 32 along k of both
+// operands is fetched once by the workgroup (thread t the 16-byte pieces t, t + 256) into one of two LDS stages while the step
+// before it is multiplied from the other; one barrier a step.  Rows of a stage are 80 bytes apart, so that the fragments'
+// reads spread over the banks.  EPI 0: relu^2, bfloat16; 1: 32-bit.
+#define MOE_LDS_ROW 40       // bfloat16 elements between rows of a stage (32 + 8)
 template <int EPI>
 __global__ void __launch_bounds__(256)
 moe_grouped_kernel(const bf16_t* __restrict__ rows, const bf16_t* __restrict__ w, const int* __restrict__ meta, int E, void* __restrict__ out,
                    int N, int K) {
+  __shared__ __attribute__((aligned(16))) bf16_t lds[2][2][128 * MOE_LDS_ROW];      // [stage][weights | rows]
   const int n_tiles = meta[0];
   if ((int)blockIdx.x >= n_tiles) return;
   const int* tile = meta + 1 + E + 1 + E + 3 * blockIdx.x;
   const int e = tile[0], row0 = tile[1], n_rows = tile[2];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r16 = lane & 15, quad = lane >> 4;
-  const int n0 = blockIdx.y * 256 + wave * 64;
-  if (n0 >= N) return;
-  // operands: lane (r16, quad) holds 8 consecutive k of row r16 of its block, from k = 8 quad on
-  const bf16_t* wa[4];
-  const bf16_t* tb[4];
-#pragma unroll
-  for (int a = 0; a < 4; ++a) wa[a] = w + ((size_t)e * N + min(n0 + 16 * a + r16, N - 1)) * K + quad * 8;
-#pragma unroll
-  for (int b = 0; b < 4; ++b) tb[b] = rows + (size_t)(row0 + min(16 * b + r16, n_rows - 1)) * K + quad * 8;
+  const int wy = wave >> 1, wx = wave & 1;
+  const int n_blk = blockIdx.y * 128;
+  // what this thread fetches: rows u / 4 of both operands, 16 bytes from element 8 (u % 4) on
+  const int u0 = threadIdx.x, u1 = threadIdx.x + 256;
+  const bf16_t* const src_w0 = w + ((size_t)e * N + min(n_blk + (u0 >> 2), N - 1)) * K + (u0 & 3) * 8;
+  const bf16_t* const src_w1 = w + ((size_t)e * N + min(n_blk + (u1 >> 2), N - 1)) * K + (u1 & 3) * 8;
+  const bf16_t* const src_r0 = rows + (size_t)(row0 + min(u0 >> 2, n_rows - 1)) * K + (u0 & 3) * 8;
+  const bf16_t* const src_r1 = rows + (size_t)(row0 + min(u1 >> 2, n_rows - 1)) * K + (u1 & 3) * 8;
+  const int park0 = (u0 >> 2) * MOE_LDS_ROW + (u0 & 3) * 8, park1 = (u1 >> 2) * MOE_LDS_ROW + (u1 & 3) * 8;
   floatx4 acc[4][4];
 #pragma unroll
   for (int a = 0; a < 4; ++a)
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[a][b] = floatx4{0.f, 0.f, 0.f, 0.f};
-  Frag8 fa[2][4], fb[2][4];
-  auto load = [&](int k, int s) {
+  uint4 w0 = *reinterpret_cast<const uint4*>(src_w0), w1 = *reinterpret_cast<const uint4*>(src_w1);
+  uint4 t0 = *reinterpret_cast<const uint4*>(src_r0), t1 = *reinterpret_cast<const uint4*>(src_r1);
+  *reinterpret_cast<uint4*>(&lds[0][0][park0]) = w0;
+  *reinterpret_cast<uint4*>(&lds[0][0][park1]) = w1;
+  *reinterpret_cast<uint4*>(&lds[0][1][park0]) = t0;
+  *reinterpret_cast<uint4*>(&lds[0][1][park1]) = t1;
+  __syncthreads();
+  int cur = 0;
+  for (int k = 0; k < K; k += 32, cur ^= 1) {       // K is a multiple of 32
+    const bool more = k + 32 < K;
+    if (more) {
+      w0 = *reinterpret_cast<const uint4*>(src_w0 + k + 32);
+      w1 = *reinterpret_cast<const uint4*>(src_w1 + k + 32);
+      t0 = *reinterpret_cast<const uint4*>(src_r0 + k + 32);
+      t1 = *reinterpret_cast<const uint4*>(src_r1 + k + 32);
+    }
+    Frag8 fa[4], fb[4];
 #pragma unroll
-    for (int a = 0; a < 4; ++a) fa[s][a].u = *reinterpret_cast<const uint4*>(wa[a] + k);
+    for (int a = 0; a < 4; ++a) fa[a].u = *reinterpret_cast<const uint4*>(&lds[cur][0][(64 * wy + 16 * a + r16) * MOE_LDS_ROW + quad * 8]);
 #pragma unroll
-    for (int b = 0; b < 4; ++b) fb[s][b].u = *reinterpret_cast<const uint4*>(tb[b] + k);
-  };
-  auto multiply = [&](int s) {
+    for (int b = 0; b < 4; ++b) fb[b].u = *reinterpret_cast<const uint4*>(&lds[cur][1][(64 * wx + 16 * b + r16) * MOE_LDS_ROW + quad * 8]);
 #pragma unroll
     for (int a = 0; a < 4; ++a)
 #pragma unroll
-      for (int b = 0; b < 4; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[s][a].v, fb[s][b].v, acc[a][b], 0, 0, 0);
-  };
-  load(0, 0);
-  for (int k = 0; k < K; k += 64) {       // K is a multiple of 32
-    if (k + 32 < K) load(k + 32, 1);
-    multiply(0);
-    if (k + 32 >= K) break;
-    if (k + 64 < K) load(k + 64, 0);
-    multiply(1);
+      for (int b = 0; b < 4; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[a].v, fb[b].v, acc[a][b], 0, 0, 0);
+    if (more) {
+      *reinterpret_cast<uint4*>(&lds[cur ^ 1][0][park0]) = w0;
+      *reinterpret_cast<uint4*>(&lds[cur ^ 1][0][park1]) = w1;
+      *reinterpret_cast<uint4*>(&lds[cur ^ 1][1][park0]) = t0;
+      *reinterpret_cast<uint4*>(&lds[cur ^ 1][1][park1]) = t1;
+    }
+    __syncthreads();
   }
-  // lane: outputs n0 + 16 a + 4 quad + i of row 16 b + r16
+  // lane: outputs n0 + 16 a + 4 quad + i of row 64 wx + 16 b + r16
+  const int n0 = n_blk + 64 * wy;
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
-    const int r = 16 * b + r16;
+    const int r = 64 * wx + 16 * b + r16;
     if (r >= n_rows) continue;
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
@@ -188,8 +205,8 @@ extern "C" int ti_moe_experts_grouped_bf16(const void* h, const int* ids, const 
   const int max_tiles = (n_pairs + MOE_TILE - 1) / MOE_TILE + E;
   moe_group_kernel<<<1, 1024, 0, stream>>>(ids, n_pairs, E, meta);
   moe_place_kernel<<<n_pairs, 128, 0, stream>>>((const bf16_t*)h, ids, wts, meta, E, top, W, scale_input, where, (bf16_t*)rows);
-  moe_grouped_kernel<0><<<dim3(max_tiles, (F + 255) / 256), 256, 0, stream>>>((const bf16_t*)rows, (const bf16_t*)up, meta, E, act, F, W);
-  moe_grouped_kernel<1><<<dim3(max_tiles, (W + 255) / 256), 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, meta, E, out, W, F);
+  moe_grouped_kernel<0><<<dim3(max_tiles, (F + 127) / 128), 256, 0, stream>>>((const bf16_t*)rows, (const bf16_t*)up, meta, E, act, F, W);
+  moe_grouped_kernel<1><<<dim3(max_tiles, (W + 127) / 128), 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, meta, E, out, W, F);
   if (y) moe_combine_kernel<<<M, 256, 0, stream>>>(out, where, y, W, top);
   TI_LAUNCH_CHECK();
   return 0;

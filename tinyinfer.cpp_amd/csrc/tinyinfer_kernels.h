@@ -192,7 +192,7 @@ int ti_moe_experts_rows(int dtype, const void* h, const int* ids, const float* w
                         float* y, int M, int W, int F, int top, int scale_input, hipStream_t stream);
 
 // ---- libti_moe_bf16: the experts for steps of many tokens, on the matrix cores: the (token, expert) pairs are laid out expert
-// by expert in tiles of 64 rows and both products run over the tiles.  Scratch: meta int32 [ti_moe_grouped_meta_ints(M top, E)],
+// by expert in tiles of 128 rows and both products run over the tiles.  Scratch: meta int32 [ti_moe_grouped_meta_ints(M top, E)],
 // where int32 [M top] (the row of every pair), rows bf16 [M top][W], act bf16 [M top][F], out f32 [M top][W].  y (may be
 // null): the tokens' sums; without it the caller adds the rows out[where[m top + k]] in ascending k.  3: sizes not served
 long ti_moe_grouped_meta_ints(int n_pairs, int E);
