@@ -2,8 +2,8 @@
 //
 //   1. moe_group: counts the (token, expert) pairs of every expert, lays the experts' runs of rows one after
 //      the other and cuts them into tiles of 128 rows: offsets, the list of tiles, cursors at zero.
-//   2. moe_place: every pair takes the next free row of its expert's run (which row does not matter: a row of
-//      a product depends on no other row) and writes its scaled input there, rounded to bfloat16.
+//   2. moe_place: every pair takes a free row of its expert's run (which row does not matter: a row of a
+//      product depends on no other row) and writes its scaled input there, rounded to bfloat16.
 //   3. two grouped products over the tiles: act = relu(A up_e^T)^2 (bfloat16), out = act down_e^T (32-bit).
 //      Weights are the A operand of v_mfma_f32_16x16x32_bf16 and tokens the 16 columns, both in their own
 //      layouts through LDS; a lane ends with four consecutive outputs of one token.
@@ -61,29 +61,48 @@ moe_group_kernel(const int* __restrict__ ids, int n_pairs, int E, int* __restric
   }
 }
 
-// a workgroup per pair: where[pair] = its row; rows[row] = bf16(s h[token]) (or h itself where the score scales the output)
-__global__ void __launch_bounds__(128)
+// A workgroup per 64 pairs: where[pair] = its row; rows[row] = bf16(s h[token]).  The workgroup counts its pairs per expert in
+// LDS and takes a run of rows from every expert's cursor at once (one atomic per expert it met, not one per pair); inside the
+// run a pair's place is its count in LDS.
+__global__ void __launch_bounds__(256)
 moe_place_kernel(const bf16_t* __restrict__ h, const int* __restrict__ ids, const float* __restrict__ wts, int* __restrict__ meta,
-                 int E, int top, int W, int scale_input, int* __restrict__ where, bf16_t* __restrict__ rows) {
-  __shared__ int s_row;
-  const int pair = blockIdx.x, m = pair / top;
-  if (threadIdx.x == 0) {
-    const int e = ids[pair];
-    const int r = meta[1 + e] + atomicAdd(&meta[1 + E + 1 + e], 1);
-    where[pair] = r;
-    s_row = r;
+                 int E, int top, int W, int n_pairs, int* __restrict__ where, bf16_t* __restrict__ rows) {
+  __shared__ int count[MOE_MAX_E];      // pairs of this workgroup per expert, then the first row of their run
+  __shared__ int s_row[64];
+  const int pair0 = blockIdx.x * 64;
+  for (int e = threadIdx.x; e < E; e += 256) count[e] = 0;
+  __syncthreads();
+  int e_mine = -1, local = 0;
+  if (threadIdx.x < 64 && pair0 + threadIdx.x < n_pairs) {
+    e_mine = ids[pair0 + threadIdx.x];
+    local = atomicAdd(&count[e_mine], 1);
   }
   __syncthreads();
-  const float s = scale_input ? wts[pair] : 1.f;
-  const bf16_t* src = h + (size_t)m * W;
-  bf16_t* dst = rows + (size_t)s_row * W;
-  for (int c = threadIdx.x * 8; c < W; c += 128 * 8) {      // W is a multiple of 32
-    const uint4 a = *reinterpret_cast<const uint4*>(src + c);
-    const unsigned w[4] = {a.x, a.y, a.z, a.w};
-    unsigned o[4];
+  for (int e = threadIdx.x; e < E; e += 256)
+    if (count[e] > 0) count[e] = meta[1 + e] + atomicAdd(&meta[1 + E + 1 + e], count[e]);
+  __syncthreads();
+  if (e_mine >= 0) {
+    const int r = count[e_mine] + local;
+    where[pair0 + threadIdx.x] = r;
+    s_row[threadIdx.x] = r;
+  }
+  __syncthreads();
+  // a wavefront copies 16 of the rows, a lane 16 bytes at a time (W is a multiple of 32)
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int i = 0; i < 16; ++i) {
+    const int pair = pair0 + wave * 16 + i;
+    if (pair >= n_pairs) break;
+    const float s = wts[pair];
+    const bf16_t* src = h + (size_t)(pair / top) * W;
+    bf16_t* dst = rows + (size_t)s_row[wave * 16 + i] * W;
+    for (int c = lane * 8; c < W; c += 64 * 8) {
+      const uint4 a = *reinterpret_cast<const uint4*>(src + c);
+      const unsigned w[4] = {a.x, a.y, a.z, a.w};
+      unsigned o[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = pack_bf16x2(__uint_as_float(w[i] << 16) * s, __uint_as_float(w[i] & 0xffff0000u) * s);
-    *reinterpret_cast<uint4*>(dst + c) = make_uint4(o[0], o[1], o[2], o[3]);
+      for (int k = 0; k < 4; ++k) o[k] = pack_bf16x2(__uint_as_float(w[k] << 16) * s, __uint_as_float(w[k] & 0xffff0000u) * s);
+      *reinterpret_cast<uint4*>(dst + c) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
   }
 }
 
@@ -204,7 +223,7 @@ extern "C" int ti_moe_experts_grouped_bf16(const void* h, const int* ids, const 
   const int n_pairs = M * top;
   const int max_tiles = (n_pairs + MOE_TILE - 1) / MOE_TILE + E;
   moe_group_kernel<<<1, 1024, 0, stream>>>(ids, n_pairs, E, meta);
-  moe_place_kernel<<<n_pairs, 128, 0, stream>>>((const bf16_t*)h, ids, wts, meta, E, top, W, scale_input, where, (bf16_t*)rows);
+  moe_place_kernel<<<(n_pairs + 63) / 64, 256, 0, stream>>>((const bf16_t*)h, ids, wts, meta, E, top, W, n_pairs, where, (bf16_t*)rows);
   moe_grouped_kernel<0><<<dim3(max_tiles, (F + 127) / 128), 256, 0, stream>>>((const bf16_t*)rows, (const bf16_t*)up, meta, E, act, F, W);
   moe_grouped_kernel<1><<<dim3(max_tiles, (W + 127) / 128), 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, meta, E, out, W, F);
   if (y) moe_combine_kernel<<<M, 256, 0, stream>>>(out, where, y, W, top);
