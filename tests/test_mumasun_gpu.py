@@ -262,6 +262,13 @@ def test_prepared_keys_and_differential_attention(ops, dtype, heads, kv, dk, dv,
                 err = np.abs(f64(fast) - want)
                 assert err.max() < bound, (shared, list(lists), np.unravel_index(err.argmax(), err.shape), err.max())
         ops.use_shared_tiles = True
+        # single tokens with a row's keys split over three workgroups, their shares merged by a kernel of its own
+        ops.force_decode_splits = 3
+        fast = torch.zeros(T, heads * dv, device="cuda", dtype=DT[dtype])
+        ops.diff_attention(*args, fast, heads, kv, dk, dv, scale, lam, eps, out_scale, block=block, all_rows=True, context=T)
+        ops.force_decode_splits = 0
+        err = np.abs(f64(fast) - want)
+        assert err.max() < bound, ("split", np.unravel_index(err.argmax(), err.shape), err.max())
         took = [c["name"] for c in ops.timing_report()]
         ops.count_calls(False)
         assert took and all("[mfma]" in n for n in took), took

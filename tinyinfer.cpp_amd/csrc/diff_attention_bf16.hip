@@ -453,7 +453,8 @@ template <int DK, int DV>
 __global__ void __launch_bounds__(256)
 diff_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool, const int* __restrict__ table, int table_stride,
                  const int* __restrict__ pos, const int* __restrict__ slot, const int* __restrict__ rows, bf16_t* __restrict__ out,
-                 int n_head, int n_kv, int P, float scale2, int block, int window, float lambda, float eps, float out_scale) {
+                 int n_head, int n_kv, int P, float scale2, int block, int window, float lambda, float eps, float out_scale,
+                 float* __restrict__ part, int n_splits) {
   extern __shared__ float lds[];     // [3 wavefronts][2 maps][DV / 4 + 2][64]
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r16 = lane & 15, quad = lane >> 4;
@@ -475,7 +476,8 @@ diff_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool, 
   MapState<DV> st[2];
   st[0].clear();
   st[1].clear();
-  walk<DK, DV>(kv, qf, lo_all / 32 + wave, p / 32 + 1, 4, lo, hi, lo_all, p, p, p, scale2, st);
+  // gridDim.z workgroups share a row's keys: workgroup z, wavefront v the pairs 4 z + v, 4 z + v + 4 gridDim.z, ...
+  walk<DK, DV>(kv, qf, lo_all / 32 + 4 * blockIdx.z + wave, p / 32 + 1, 4 * n_splits, lo, hi, lo_all, p, p, p, scale2, st);
   constexpr int PER_MAP = (DV / 4 + 2) * 64;
   if (wave > 0) {
     float* mine = lds + (size_t)(wave - 1) * 2 * PER_MAP;
@@ -494,6 +496,55 @@ diff_rows_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool, 
   if (wave > 0) return;
   for (int w = 0; w < 3; ++w) {
     const float* theirs = lds + (size_t)w * 2 * PER_MAP;
+#pragma unroll
+    for (int mp = 0; mp < 2; ++mp) {
+      const float* src = theirs + mp * PER_MAP;
+      const float m2 = src[DV / 4 * 64 + lane], l2 = src[(DV / 4 + 1) * 64 + lane];
+      const float mm = fmaxf(st[mp].m, m2);
+      const float m_safe = (mm == -INFINITY) ? 0.f : mm;
+      const float a = __builtin_amdgcn_exp2f(st[mp].m - m_safe), b = __builtin_amdgcn_exp2f(m2 - m_safe);
+      st[mp].l = st[mp].l * a + l2 * b;
+#pragma unroll
+      for (int d = 0; d < DV / 16; ++d)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) st[mp].o[d][i] = st[mp].o[d][i] * a + src[(d * 4 + i) * 64 + lane] * b;
+      st[mp].m = mm;
+    }
+  }
+  if (n_splits == 1) {
+    finish_column<DV>(st, lambda, eps, out_scale, out + ((size_t)m * n_head + h) * DV, live);
+    return;
+  }
+  // the workgroup's share goes to memory as it lies in the lanes; diff_rows_merge_kernel adds the shares up
+  float* mine = part + (((size_t)blockIdx.x * n_kv + kvh) * n_splits + blockIdx.z) * 2 * PER_MAP;
+#pragma unroll
+  for (int mp = 0; mp < 2; ++mp) {
+    float* dstp = mine + mp * PER_MAP;
+#pragma unroll
+    for (int d = 0; d < DV / 16; ++d)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dstp[(d * 4 + i) * 64 + lane] = st[mp].o[d][i];
+    dstp[DV / 4 * 64 + lane] = st[mp].m;
+    dstp[(DV / 4 + 1) * 64 + lane] = st[mp].l;
+  }
+}
+
+// one wavefront per (row, kv head): the shares of the workgroups that split the row's keys, in ascending order
+template <int DV>
+__global__ void __launch_bounds__(64)
+diff_rows_merge_kernel(const float* __restrict__ part, const int* __restrict__ rows, bf16_t* __restrict__ out, int n_head, int n_kv,
+                       int n_splits, float lambda, float eps, float out_scale) {
+  constexpr int PER_MAP = (DV / 4 + 2) * 64;
+  const int lane = threadIdx.x, r16 = lane & 15;
+  const int m = rows ? rows[blockIdx.x] : blockIdx.x;
+  const int kvh = blockIdx.y, per = n_head / n_kv;
+  const bool live = r16 < per;
+  const int h = kvh * per + (live ? r16 : 0);
+  MapState<DV> st[2];
+  st[0].clear();
+  st[1].clear();
+  for (int s = 0; s < n_splits; ++s) {
+    const float* theirs = part + (((size_t)blockIdx.x * n_kv + kvh) * n_splits + s) * 2 * PER_MAP;
 #pragma unroll
     for (int mp = 0; mp < 2; ++mp) {
       const float* src = theirs + mp * PER_MAP;
@@ -563,22 +614,35 @@ extern "C" int ti_diff_attention_tiles_bf16(const void* q, const void* pool, con
 extern "C" int ti_diff_attention_rows_bf16(const void* q, const void* pool, const int* table, int table_stride, const int* pos,
                                            const int* slot, const int* rows, void* out, int n_rows, int n_head, int n_kv, int dk,
                                            int dv, int page_size, float scale, int block, int window, float lambda, float eps,
-                                           float out_scale, hipStream_t stream) {
+                                           float out_scale, float* part, int n_splits, hipStream_t stream) {
   if (!served(dk, dv, page_size, n_head, n_kv) || n_head / n_kv > 16) {
     ti_set_error("diff_attention (rows): sizes %d / %d, pages of %d, %d heads a kv head are not served", dk, dv, page_size,
                  n_kv > 0 ? n_head / n_kv : 0);
     return 3;
   }
   TI_REQUIRE(n_kv <= 65535 && table_stride > 0 && block >= 0 && window >= 0, "diff_attention (rows): bad arguments");
+  TI_REQUIRE(n_splits >= 1 && n_splits <= 64 && (n_splits == 1 || part), "diff_attention (rows): %d splits need scratch", n_splits);
   if (n_rows == 0) return 0;
-  dim3 grid(n_rows, n_kv);
+  dim3 grid(n_rows, n_kv, n_splits);
   const size_t lds = (size_t)3 * 2 * (dv / 4 + 2) * 64 * 4;
 #define DA_ROWS(K, V)                                                                                                             \
   diff_rows_kernel<K, V><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table, table_stride, pos, slot, rows, \
                                                      (bf16_t*)out, n_head, n_kv, page_size, scale * DA_LOG2E, block, window,      \
-                                                     lambda, eps, out_scale)
+                                                     lambda, eps, out_scale, part, n_splits)
   DA_DISPATCH(DA_ROWS);
 #undef DA_ROWS
   TI_LAUNCH_CHECK();
+  if (n_splits > 1) {
+    const dim3 mgrid(n_rows, n_kv);
+    if (dv == 32) diff_rows_merge_kernel<32><<<mgrid, 64, 0, stream>>>(part, rows, (bf16_t*)out, n_head, n_kv, n_splits, lambda, eps, out_scale);
+    else if (dv == 64) diff_rows_merge_kernel<64><<<mgrid, 64, 0, stream>>>(part, rows, (bf16_t*)out, n_head, n_kv, n_splits, lambda, eps, out_scale);
+    else diff_rows_merge_kernel<128><<<mgrid, 64, 0, stream>>>(part, rows, (bf16_t*)out, n_head, n_kv, n_splits, lambda, eps, out_scale);
+    TI_LAUNCH_CHECK();
+  }
   return 0;
+}
+
+// floats of scratch for ti_diff_attention_rows_bf16 with n_splits > 1
+extern "C" long ti_diff_attention_rows_scratch(int n_rows, int n_kv, int dv, int n_splits) {
+  return (long)n_rows * n_kv * n_splits * 2 * (dv / 4 + 2) * 64;
 }

@@ -174,11 +174,14 @@ int ti_diff_attention_tiles_bf16(const void* q, const void* pool, const int* tab
                                  int page_size, float scale, int block, int window, float lambda, float eps, float out_scale,
                                  int use_lds, hipStream_t stream);
 // (use_lds 1: the four wavefronts of a tile share the keys and values they read through LDS; 0: each fetches its own)
-// single rows (rows int32 [n_rows], or null: rows 0 .. n_rows - 1); at most 16 query heads a kv head
+// single rows (rows int32 [n_rows], or null: rows 0 .. n_rows - 1); at most 16 query heads a kv head.  n_splits > 1: so many
+// workgroups share a row's keys and leave their shares in part (f32, ti_diff_attention_rows_scratch floats) for a kernel that
+// merges them
 int ti_diff_attention_rows_bf16(const void* q, const void* pool, const int* table, int table_stride, const int* pos,
                                 const int* slot, const int* rows, void* out, int n_rows, int n_head, int n_kv, int dk, int dv,
                                 int page_size, float scale, int block, int window, float lambda, float eps, float out_scale,
-                                hipStream_t stream);
+                                float* part, int n_splits, hipStream_t stream);
+long ti_diff_attention_rows_scratch(int n_rows, int n_kv, int dv, int n_splits);
 
 // ---- libti_moe: a mixture of experts
 // scores (score_kind 0: sigmoid, 1: softmax over the experts) of h [M, W] against router f32 [E, W] in 32-bit; the `top`

@@ -1305,6 +1305,10 @@ int ti_ops_call(void* ops_, const char* op_, const ti_tensor* t, int n_t, const 
       l.n_rows = (int)num(10);
     }
     if (n_t > 8) l.entry_meta = iptr(8);
+    if (n_s > 11) {      // the longest context of a single row: its keys may be split over workgroups
+      l.context = (int)num(11);
+      l.ws = &workspace_of(&ops);
+    }
     ops.diff_attention(arg(0), arg(1), view_of(2, arg(1)), iptr(3), iptr(4), arg(5), (int)num(0), (int)num(1), (int)num(2), (int)num(3),
                        (float)num(4), (int)num(5), (int)num(6), (float)num(7), (float)num(8), (float)num(9), listed ? &l : nullptr);
   } else if (op == "moe_route") {

@@ -372,8 +372,10 @@ class Ops {
   // lists (device int32, the step's metadata): tiles [n_tiles][3] = (entry, first row, rows <= 64) of the entries of several
   // tokens, rows [n_rows] the rows of single-token entries (null with n_rows = M: every row is one).  With them the bfloat16
   // matrix-core kernels serve the sizes they take; without, or for other sizes and float32, every row is walked on its own
+  // context: the longest context a single row reads (what the split of its keys over workgroups is sized for; 0: no split);
+  // ws: where the shares of a split go
   struct DiffAttentionLists { const int* tiles = nullptr; int n_tiles = 0; const int* rows = nullptr; int n_rows = 0;
-                              const int* entry_meta = nullptr; };
+                              const int* entry_meta = nullptr; int context = 0; Workspace* ws = nullptr; };
   void diff_attention(const Tensor& q, const Tensor& pool, const CacheView& view, const int* positions, const int* slots,
                       const Tensor& out, int heads, int kv_heads, int dk, int dv, float scale, int block, int window, float lambda,
                       float eps, float out_scale, const DiffAttentionLists* lists = nullptr);
@@ -416,7 +418,7 @@ class Ops {
     bool radix_sample = true;       // draws with a top-k cut: many workgroups share a row (else one walks it bit by bit)
     bool shared_tiles = true;       // differential attention over a portion: a tile's wavefronts share keys and values through LDS
     int force_paired_tiles = -1;    // 1 / 0: that kernel with / without pairs, whatever the launch
-    int force_decode_splits = 0;    // > 0: the decode attention cuts every context into this many runs
+    int force_decode_splits = 0;    // > 0: the decode attention cuts every context into this many runs (differential attention too)
   } use;
   // A shape rule of a kernel library forced for this object's calls (tests and measurements; the names are listed
   // in csrc/tinyinfer_kernels_tuning.h).  The rules are the libraries' own, process-wide: this object sets its

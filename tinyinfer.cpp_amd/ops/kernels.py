@@ -382,7 +382,7 @@ class Ops:
         self._call("diff_qk_prep", tensors, [eps, heads, kv_heads, dk, dv, rot_dims, mag])
 
     def diff_attention(self, q, pool, table, positions, slots, out, heads, kv_heads, dk, dv, scale, lam, eps, out_scale, block=0, window=0,
-                       tiles=None, rows=None, entries=None, all_rows=False):
+                       tiles=None, rows=None, entries=None, all_rows=False, context=0):
         """tiles int32 [n, 3] = (entry, first row, rows <= 64) with entries int32 [R, 4] = (row0, tokens, start, -), rows int32 [n]
         (or all_rows: every row is a single token): the lists of the bfloat16 matrix-core kernels; without them every row is
         walked on its own."""
@@ -390,8 +390,9 @@ class Ops:
         libs = ["diff_attention"]
         if tiles is not None or rows is not None or all_rows:
             tensors += [tiles, rows, entries]
-            if all_rows:
-                numbers.append(q.shape[0])
+            numbers.append(q.shape[0] if all_rows else 0)
+            if context:
+                numbers.append(context)        # the longest context of a single row: its keys may be split over workgroups
             if q.dtype == native.torch().bfloat16:
                 libs.append("diff_attention_bf16")
         self._call("diff_attention", tensors, numbers, libs=libs)

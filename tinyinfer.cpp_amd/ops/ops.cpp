@@ -1095,11 +1095,28 @@ void Ops::diff_attention(const Tensor& q, const Tensor& pool, const CacheView& v
                                                                        lists->entry_meta, out.data, lists->n_tiles, heads, kv_heads, dk,
                                                                        dv, (int)pool.shape[2], scale, block, window, lambda, eps,
                                                                        out_scale, use.shared_tiles ? 1 : 0, (hipStream_t)launch_stream());
-    if (rc == 0 && lists->n_rows)
+    if (rc == 0 && lists->n_rows) {
+      // few rows and long contexts: several workgroups share a row's keys, until about one workgroup a compute unit runs and
+      // a wavefront still walks four pairs of blocks
+      int reach = lists->context;
+      if (block > 0) reach = std::min(reach, block);
+      if (window > 0) reach = std::min(reach, window);
+      int splits = 1;
+      if (lists->ws && reach > 0) {
+        const int by_units = compute_units() / std::max(1, lists->n_rows * kv_heads);
+        splits = std::max(1, std::min({8, by_units, reach / (32 * 16)}));
+      }
+      if (use.force_decode_splits > 0 && lists->ws) splits = std::min(64, use.force_decode_splits);
+      float* part = nullptr;
+      if (splits > 1) {
+        const long floats = KERNEL("diff_attention_bf16", ti_diff_attention_rows_scratch)(lists->n_rows, kv_heads, dv, splits);
+        part = (float*)lists->ws->get("dattn.part", (size_t)floats * 4);
+      }
       rc = KERNEL("diff_attention_bf16", ti_diff_attention_rows_bf16)(q.data, pool.data, view.table, view.table_width, positions, slots,
                                                                       lists->rows, out.data, lists->n_rows, heads, kv_heads, dk, dv,
                                                                       (int)pool.shape[2], scale, block, window, lambda, eps, out_scale,
-                                                                      (hipStream_t)launch_stream());
+                                                                      part, splits, (hipStream_t)launch_stream());
+    }
     if (rc == 0) {
       took("[mfma]");
       return;

@@ -1441,6 +1441,9 @@ class DiffAttention final : public MixerPart {
   Ops::DiffAttentionLists lists(const StepContext& ctx) const {
     Ops::DiffAttentionLists l;
     l.entry_meta = ctx.entry_meta;
+    // a captured graph serves every later step of its shape: what it launches is sized for the longest sequence
+    l.context = ctx.plan && ctx.plan->sized_for_longest() ? ctx.plan->max_seq() : ctx.max_context;
+    l.ws = &ctx.ws;
     if (ctx.decode_only) {
       l.n_rows = (int)ctx.M;
       return l;
