@@ -143,88 +143,203 @@ extern "C" int ti_moe_route(int dtype, const void* h, const float* router, int* 
 }
 
 // ------------------------------------------------------------ the experts, an output a wavefront
-// up [E][F][W], down [E][W][F] in T.  Two kernels: act[(m, k)][f] = relu(up[e_k][f] . (s_k h[m]))^2 rounded to T, for every
-// token m and chosen expert k; then y[m][c] = sum_k down[e_k][c] . act[(m, k)], k ascending.  A wavefront owns ROWS outputs;
-// its lanes share a row of the weight in pieces of 16 bytes (lane l the pieces l, l + 64, ... in ascending order, then a
-// butterfly): the order of every sum is fixed, whatever else the step holds.
+// up [E][F][W], down [E][W][F] in T.  Two kernels, both with a workgroup per (expert, 16 outputs): the workgroup finds the
+// pairs (token, choice) of its expert, NP at a time, keeps their input rows in LDS and walks its rows of the weight once for
+// all of them: an expert's weights are read once a step however many tokens chose it.
+//   act[pair][f] = relu(up[e][f] . (s h[token]))^2 rounded to T;   part[pair][c] = down[e][c] . act[pair]
+// and a token's rows of `part` are added in the order its experts were chosen by whoever reads them (moe_sum_pairs, or the
+// norm that follows).  A wavefront owns four outputs; its lanes share a row of the weight in pieces of 16 bytes (lane l the
+// pieces l, l + 64, ... in ascending order, then a butterfly): the order of every sum is fixed, whatever else the step holds.
 #define MOE_ROWS 4      // outputs a wavefront
-template <typename T, bool VEC>
-__global__ void __launch_bounds__(256)
-moe_up_rows_kernel(const T* __restrict__ h, const int* __restrict__ ids, const float* __restrict__ wts, const T* __restrict__ up,
-                   T* __restrict__ act, int W, int F, int top, int scale_input) {
-  extern __shared__ float hs[];      // [W] the expert's input
-  const int pair = blockIdx.x, m = pair / top;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int e = ids[pair];
-  const float s = wts[pair];
-  for (int c = threadIdx.x; c < W; c += 256) {
-    const float v = ld<T>(h + (size_t)m * W + c);
-    float r = scale_input ? v * s : v;
-    if (sizeof(T) == 2) r = bf2f(f2bf(r));
-    hs[c] = r;
-  }
-  __syncthreads();
-  const int f0 = (blockIdx.y * 4 + wave) * MOE_ROWS;
-  const T* wu = up + (size_t)e * F * W;
-#pragma unroll
-  for (int r = 0; r < MOE_ROWS; ++r) {
-    const int f = f0 + r;
-    if (f >= F) break;
-    const float z = wave_dot<T, VEC>([&](int c) { return hs[c]; }, wu + (size_t)f * W, W, lane);
-    if (lane == 0) {
-      float a = fmaxf(z, 0.f);
-      st<T>(act + (size_t)pair * F + f, a * a);
+
+// the next pairs of expert e from pair `next` on, at most NP: their indices to s_pairs, (count, where to go on) to s_found.
+// Called by the first wavefront.
+template <int NP>
+__device__ __forceinline__ void next_pairs(const int* __restrict__ ids, int n_pairs, int e, int next, int* s_pairs, int* s_found) {
+  const int lane = threadIdx.x & 63;
+  int n = 0, i = next;
+  while (i < n_pairs && n < NP) {
+    const bool hit = i + lane < n_pairs && ids[i + lane] == e;
+    unsigned long long mask = __ballot(hit);
+    int consumed = 64;
+    while (mask) {
+      const int b = __ffsll((long long)mask) - 1;
+      if (n == NP) {       // this one waits for the next round
+        consumed = b;
+        break;
+      }
+      if (lane == 0) s_pairs[n] = i + b;
+      ++n;
+      mask &= mask - 1;
     }
+    i += consumed;
+  }
+  if (lane == 0) {
+    s_found[0] = n;
+    s_found[1] = i;
   }
 }
 
-template <typename T, bool VEC>
+// z[r][p] = rows[p] . b[r] for the NP rows in LDS (T) and MOE_ROWS rows of the weight in memory, K apart (rows of the weight
+// beyond the last one are read as the last one): the loads of all the weight's rows are in flight together.  Every sum runs
+// over a lane's pieces in ascending order, then a butterfly.
+template <typename T, bool VEC, int NP>
+__device__ __forceinline__ void wave_dots(const T* rows, int n_live, const T* __restrict__ b, int n_rows_w, int K, int lane,
+                                          float (*z)[NP]) {
+#pragma unroll
+  for (int r = 0; r < MOE_ROWS; ++r)
+#pragma unroll
+    for (int p = 0; p < NP; ++p) z[r][p] = 0.f;
+  const T* br[MOE_ROWS];
+#pragma unroll
+  for (int r = 0; r < MOE_ROWS; ++r) br[r] = b + (size_t)(r < n_rows_w ? r : n_rows_w - 1) * K;
+  if (VEC) {
+    constexpr int N = Piece<T>::N;
+    for (int c = lane * N; c < K; c += 64 * N) {
+      float v[MOE_ROWS][N];
+#pragma unroll
+      for (int r = 0; r < MOE_ROWS; ++r) Piece<T>::load(br[r] + c, v[r]);
+#pragma unroll
+      for (int p = 0; p < NP; ++p)
+        if (p < n_live) {
+          float a[N];
+          Piece<T>::load(rows + (size_t)p * K + c, a);
+#pragma unroll
+          for (int r = 0; r < MOE_ROWS; ++r)
+#pragma unroll
+            for (int i = 0; i < N; ++i) z[r][p] = fmaf(a[i], v[r][i], z[r][p]);
+        }
+    }
+  } else {
+    for (int c = lane; c < K; c += 64) {
+      float v[MOE_ROWS];
+#pragma unroll
+      for (int r = 0; r < MOE_ROWS; ++r) v[r] = ld<T>(br[r] + c);
+#pragma unroll
+      for (int p = 0; p < NP; ++p)
+        if (p < n_live) {
+          const float a = ld<T>(rows + (size_t)p * K + c);
+#pragma unroll
+          for (int r = 0; r < MOE_ROWS; ++r) z[r][p] = fmaf(a, v[r], z[r][p]);
+        }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < MOE_ROWS; ++r)
+#pragma unroll
+    for (int p = 0; p < NP; ++p) z[r][p] = group_sum<64>(z[r][p]);
+}
+
+// DOWN false: rows are the tokens' inputs h (scaled by the score where it scales the input), K = W, outputs F, relu^2 to act.
+// DOWN true: rows are act, K = F, outputs W, 32-bit to part (times the score where it scales the output).
+template <typename T, bool VEC, int NP, bool DOWN>
 __global__ void __launch_bounds__(256)
-moe_down_rows_kernel(const T* __restrict__ act, const int* __restrict__ ids, const float* __restrict__ wts, const T* __restrict__ down,
-                     float* __restrict__ y, int W, int F, int top, int scale_input) {
+moe_expert_rows_kernel(const T* __restrict__ in, const int* __restrict__ ids, const float* __restrict__ wts, const T* __restrict__ w,
+                       void* __restrict__ out, int n_pairs, int K, int N, int top, int scale_input) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char raw[];
+  T* rows = reinterpret_cast<T*>(raw);      // [NP][K]
+  __shared__ int s_pairs[NP], s_found[2];
+  const int e = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int n0 = (blockIdx.y * 4 + wave) * MOE_ROWS;
+  const T* we = w + (size_t)e * N * K;
+  int next = 0;
+  while (next < n_pairs) {
+    if (wave == 0) next_pairs<NP>(ids, n_pairs, e, next, s_pairs, s_found);
+    __syncthreads();
+    const int n_live = s_found[0];
+    next = s_found[1];
+    if (n_live == 0) break;
+    for (int p = 0; p < n_live; ++p) {
+      const int pair = s_pairs[p];
+      const T* src = DOWN ? in + (size_t)pair * K : in + (size_t)(pair / top) * K;
+      const float s = (!DOWN && scale_input) ? wts[pair] : 1.f;
+      for (int c = threadIdx.x; c < K; c += 256) st<T>(rows + (size_t)p * K + c, DOWN ? ld<T>(src + c) : ld<T>(src + c) * s);
+    }
+    __syncthreads();
+    if (n0 < N) {
+      float z[MOE_ROWS][NP];
+      const int n_rows_w = min(MOE_ROWS, N - n0);
+      wave_dots<T, VEC, NP>(rows, n_live, we + (size_t)n0 * K, n_rows_w, K, lane, z);
+      if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < MOE_ROWS; ++r)
+#pragma unroll
+          for (int p = 0; p < NP; ++p)
+            if (r < n_rows_w && p < n_live) {
+              const int pair = s_pairs[p], n = n0 + r;
+              if (DOWN) {
+                ((float*)out)[(size_t)pair * N + n] = scale_input ? z[r][p] : z[r][p] * wts[pair];
+              } else {
+                const float a = fmaxf(z[r][p], 0.f);
+                st<T>((T*)out + (size_t)pair * N + n, a * a);
+              }
+            }
+      }
+    }
+    __syncthreads();      // the rows and the list are read to the end before the next round writes them
+  }
+}
+
+// y[m] = sum_k part[m top + k], k ascending
+__global__ void moe_sum_pairs_kernel(const float* __restrict__ part, float* __restrict__ y, int W, int top) {
   const int m = blockIdx.x;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int c0 = (blockIdx.y * 4 + wave) * MOE_ROWS;
-#pragma unroll
-  for (int r = 0; r < MOE_ROWS; ++r) {
-    const int c = c0 + r;
-    if (c >= W) break;
-    float acc = 0.f;
-    for (int k = 0; k < top; ++k) {
-      const int pair = m * top + k;
-      const T* a = act + (size_t)pair * F;
-      const T* wd = down + ((size_t)ids[pair] * W + c) * F;
-      float z = wave_dot<T, VEC>([&](int f) { return ld<T>(a + f); }, wd, F, lane);
-      if (!scale_input) z *= wts[pair];
-      acc = k == 0 ? z : acc + z;
-    }
-    if (lane == 0) y[(size_t)m * W + c] = acc;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float v = part[(size_t)m * top * W + c];
+    for (int k = 1; k < top; ++k) v += part[((size_t)m * top + k) * W + c];
+    y[(size_t)m * W + c] = v;
   }
 }
 
-// act: scratch in the dtype of h, [M top][F]
+template <typename T, bool VEC, int NP, bool DOWN>
+static void launch_expert_rows(const void* in, const int* ids, const float* wts, const void* w, void* out, int n_pairs, int K, int N,
+                               int top, int scale_input, int E, hipStream_t stream) {
+  const dim3 grid(E, (N + 4 * MOE_ROWS - 1) / (4 * MOE_ROWS));
+  moe_expert_rows_kernel<T, VEC, NP, DOWN><<<grid, 256, (size_t)NP * K * sizeof(T), stream>>>((const T*)in, ids, wts, (const T*)w, out,
+                                                                                               n_pairs, K, N, top, scale_input);
+}
+template <typename T, bool VEC, bool DOWN>
+static int expert_rows(const void* in, const int* ids, const float* wts, const void* w, void* out, int n_pairs, int K, int N, int top,
+                       int scale_input, int E, hipStream_t stream) {
+  const size_t row = (size_t)K * sizeof(T), room = 48 * 1024;      // rows of the pairs a round holds in LDS
+  if (4 * row <= room) launch_expert_rows<T, VEC, 4, DOWN>(in, ids, wts, w, out, n_pairs, K, N, top, scale_input, E, stream);
+  else if (2 * row <= room) launch_expert_rows<T, VEC, 2, DOWN>(in, ids, wts, w, out, n_pairs, K, N, top, scale_input, E, stream);
+  else if (row <= 64 * 1024) launch_expert_rows<T, VEC, 1, DOWN>(in, ids, wts, w, out, n_pairs, K, N, top, scale_input, E, stream);
+  else return 1;
+  return 0;
+}
+
+// act: scratch in the dtype of h, [M top][F]; part: f32 [M top][W], a token's rows to be added in ascending order: into y where
+// y is given, else by the caller
 extern "C" int ti_moe_experts_rows(int dtype, const void* h, const int* ids, const float* wts, const void* up, const void* down,
-                                   void* act, float* y, int M, int W, int F, int top, int scale_input, hipStream_t stream) {
-  TI_REQUIRE(M >= 0 && W > 0 && F > 0 && top > 0, "moe_experts: bad sizes M=%d W=%d F=%d top=%d", M, W, F, top);
-  TI_REQUIRE((size_t)W * 4 <= 64 * 1024, "moe_experts: a width of %d does not fit the workgroup's 64 KB", W);
+                                   void* act, float* part, float* y, int M, int W, int F, int E, int top, int scale_input,
+                                   hipStream_t stream) {
+  TI_REQUIRE(M >= 0 && W > 0 && F > 0 && top > 0 && E > 0, "moe_experts: bad sizes M=%d W=%d F=%d top=%d", M, W, F, top);
   if (M == 0) return 0;
-  const size_t lds = (size_t)W * 4;
-  const dim3 up_grid(M * top, (F + 4 * MOE_ROWS - 1) / (4 * MOE_ROWS)), down_grid(M, (W + 4 * MOE_ROWS - 1) / (4 * MOE_ROWS));
-  TI_REQUIRE(up_grid.y <= 65535 && down_grid.y <= 65535, "moe_experts: sizes W=%d F=%d are too large", W, F);
-  const size_t es = dtype == TI_F32 ? 4 : 2;
-  const int piece = (int)(16 / es);
-  const bool vec = W % piece == 0 && F % piece == 0 && (((uintptr_t)up | (uintptr_t)down | (uintptr_t)act) & 15) == 0;
-#define MOE_LAUNCH(T, V)                                                                                                              do {                                                                                                                                  moe_up_rows_kernel<T, V><<<up_grid, 256, lds, stream>>>((const T*)h, ids, wts, (const T*)up, (T*)act, W, F, top, scale_input);      moe_down_rows_kernel<T, V><<<down_grid, 256, 0, stream>>>((const T*)act, ids, wts, (const T*)down, y, W, F, top, scale_input);    } while (0)
+  TI_REQUIRE((F + 4 * MOE_ROWS - 1) / (4 * MOE_ROWS) <= 65535 && (W + 4 * MOE_ROWS - 1) / (4 * MOE_ROWS) <= 65535,
+             "moe_experts: sizes W=%d F=%d are too large", W, F);
+  const int es = dtype == TI_F32 ? 4 : 2;
+  const int piece = 16 / es;
+  const bool vec = W % piece == 0 && F % piece == 0 && (((uintptr_t)up | (uintptr_t)down | (uintptr_t)act | (uintptr_t)h) & 15) == 0;
+  const int n_pairs = M * top;
+  int rc;
+#define MOE_BOTH(T, V)                                                                                              \
+  do {                                                                                                              \
+    rc = expert_rows<T, V, false>(h, ids, wts, up, act, n_pairs, W, F, top, scale_input, E, stream);                \
+    if (rc == 0) rc = expert_rows<T, V, true>(act, ids, wts, down, part, n_pairs, F, W, top, scale_input, E, stream); \
+  } while (0)
   if (dtype == TI_F32) {
-    if (vec) MOE_LAUNCH(float, true);
-    else MOE_LAUNCH(float, false);
+    if (vec) MOE_BOTH(float, true);
+    else MOE_BOTH(float, false);
   } else if (dtype == TI_BF16) {
-    if (vec) MOE_LAUNCH(bf16_t, true);
-    else MOE_LAUNCH(bf16_t, false);
+    if (vec) MOE_BOTH(bf16_t, true);
+    else MOE_BOTH(bf16_t, false);
   } else {
     TI_REQUIRE(false, "moe_experts: unknown dtype %d", dtype);
   }
-#undef MOE_LAUNCH
+#undef MOE_BOTH
+  TI_REQUIRE(rc == 0, "moe_experts: a row of %d or %d entries does not fit the workgroup's 64 KB", W, F);
+  if (y) moe_sum_pairs_kernel<<<M, 256, 0, stream>>>(part, y, W, top);
   TI_LAUNCH_CHECK();
   return 0;
 }

@@ -7,7 +7,8 @@
 TI_ERROR_API
 
 // x[m] (+)= y'[m] / sqrt(mean(y'[m]^2) + eps) * g, with y'[m] = y[m], or, with `gather`, the sum of the
-// n_gather rows y[gather[m n_gather + k]] in ascending k (the rows a token's experts left).
+// n_gather rows y[gather[m n_gather + k]] in ascending k (the rows a token's experts left; without a list: the rows
+// y[m n_gather + k]).
 // A workgroup per row; each thread owns the elements t, t + 256, ... in both passes, so y and x may be
 // the same memory.  The sum of squares: per thread in ascending order, then block_sum (fixed order).
 // RT: also `rounded` (RT) [M][H] = the new x rounded, for the product that reads the residual next.
@@ -18,9 +19,12 @@ norm_residual_kernel(float* __restrict__ x, const float* __restrict__ y, const f
   __shared__ float red[4];
   const int m = blockIdx.x;
   auto value = [&](int i) {
-    if (!gather) return y[(size_t)m * H + i];
+    if (n_gather <= 1 && !gather) return y[(size_t)m * H + i];
     float v = 0.f;
-    for (int k = 0; k < n_gather; ++k) v += y[(size_t)gather[(size_t)m * n_gather + k] * H + i];
+    for (int k = 0; k < n_gather; ++k) {
+      const size_t r = gather ? (size_t)gather[(size_t)m * n_gather + k] : (size_t)m * n_gather + k;
+      v = k == 0 ? y[r * H + i] : v + y[r * H + i];
+    }
     return v;
   };
   float ss = 0.f;

@@ -134,7 +134,7 @@ int ti_gated_head_norm(int out_dtype, const float* o, const float* gate, int ld,
 
 // ---- libti_residual: layers that norm what a sublayer returns
 // x[m] (+)= y'[m] / sqrt(mean(y'[m]^2) + eps) * g; y'[m] = y[m], or with `gather` (int32 [M][n_gather]) the sum of
-// the rows y[gather[m][k]] in ascending k.  accumulate 0: x is overwritten (y may be x itself).  rounded (may be null):
+// the rows y[gather[m][k]] in ascending k (gather null and n_gather > 1: of the rows y[m n_gather + k]).  accumulate 0: x is overwritten (y may be x itself).  rounded (may be null):
 // [M][H] of rounded_dtype, the new x rounded for the product that reads it next
 int ti_norm_residual(float* x, const float* y, const float* g, const int* gather, int n_gather, int M, int H, float eps,
                      int accumulate, void* rounded, int rounded_dtype, hipStream_t stream);
@@ -189,10 +189,11 @@ long ti_diff_attention_rows_scratch(int n_rows, int n_kv, int dv, int n_splits);
 int ti_moe_route(int dtype, const void* h, const float* router, int* ids, float* wts, int M, int W, int E, int top,
                  int score_kind, int renormalize, hipStream_t stream);
 // y f32 [M, W] = sum_k down[e_k] relu(up[e_k] (s_k h))^2 (scale_input) or sum_k s_k down[e_k] relu(up[e_k] h)^2;
-// up [E][F][W], down [E][W][F] in the dtype of h; act: scratch of that dtype, [M top][F].  An output a wavefront: steps of
-// few tokens, and float32
+// up [E][F][W], down [E][W][F] in the dtype of h; act: scratch of that dtype, [M top][F]; part: f32 [M top][W].  A workgroup
+// per expert and 16 outputs walks its weights once for all the pairs that chose the expert: steps of few tokens, and float32.
+// A token's rows of part are added in ascending order into y where y is given, else left to the caller
 int ti_moe_experts_rows(int dtype, const void* h, const int* ids, const float* wts, const void* up, const void* down, void* act,
-                        float* y, int M, int W, int F, int top, int scale_input, hipStream_t stream);
+                        float* part, float* y, int M, int W, int F, int E, int top, int scale_input, hipStream_t stream);
 
 // ---- libti_moe_bf16: the experts for steps of many tokens, on the matrix cores: the (token, expert) pairs are laid out expert
 // by expert in tiles of 128 rows and both products run over the tiles.  Scratch: meta int32 [ti_moe_grouped_meta_ints(M top, E)],

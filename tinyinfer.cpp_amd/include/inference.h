@@ -350,7 +350,8 @@ class Ops {
                        int heads, int dv);
   // ---- layers that norm what a sublayer returns; short convolutions; differential attention; mixtures of experts
   // x (+)= y / rms(y) * gain (32-bit; gain is the factor itself).  accumulate false: x is overwritten (y may be x).
-  // gather (device int32 [M][n_gather]): row m of y is the sum of the rows y[gather[m][k]], k ascending
+  // gather (device int32 [M][n_gather]): row m of y is the sum of the rows y[gather[m][k]], k ascending; no list and
+  // n_gather > 1: of the rows y[m n_gather + k]
   // rounded (may be null): also receives the new x in its own dtype, for the product that reads the residual next
   void norm_residual(const Tensor& x, const Tensor& y, const Tensor& gain, float eps, bool accumulate, const int* gather = nullptr,
                      int n_gather = 0, const Tensor* rounded = nullptr);
@@ -386,7 +387,8 @@ class Ops {
   // y f32 [M, W] = sum over a token's experts of down_e relu(up_e h)^2, the weight on the expert's input or output;
   // up [E F, W], down [E W, F]; scratch comes from `ws`.  With `rows` (and bfloat16, many tokens, sizes the matrix-core kernels
   // take) y may stay unwritten: then rows->t is f32 [M top, W] and rows->gather device int32 [M][top]: row m of the result is
-  // the sum of the rows rows->t[gather[m][k]], k ascending, left to the norm that reads it (Ops::norm_residual)
+  // the sum of the rows rows->t[gather[m][k]], k ascending (no list: of the rows m n_gather + k), left to the norm that
+  // reads it (Ops::norm_residual)
   struct GatheredRows { Tensor t; const int* gather = nullptr; int n_gather = 0; };
   void moe_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, const Tensor& up, const Tensor& down, const Tensor& y,
                    int experts, bool scale_input, Workspace& ws, GatheredRows* rows = nullptr);

@@ -999,7 +999,8 @@ void Ops::norm_residual(const Tensor& x, const Tensor& y, const Tensor& gain, fl
   TIMED("norm_residual " + dims(x));
   const int64_t H = x.ndim == 2 ? x.shape[1] : 0;
   require(x.ndim == 2 && x.dtype == DType::F32 && x.contiguous() && y.ndim == 2 && y.dtype == DType::F32 && y.contiguous() &&
-              y.shape[1] == H && (gather ? n_gather > 0 : y.shape[0] == x.shape[0]) && gain.dtype == DType::F32 && gain.numel() == H,
+              y.shape[1] == H && (gather ? n_gather > 0 : y.shape[0] == x.shape[0] * std::max(1, n_gather)) &&
+              gain.dtype == DType::F32 && gain.numel() == H,
           "norm_residual: x " + x.describe() + ", y " + y.describe() + " or gain " + gain.describe() + " do not fit");
   require(!rounded || (rounded->contiguous() && rounded->numel() == x.numel()), "norm_residual: the rounded copy does not fit x");
   int rc = KERNEL("residual", ti_norm_residual)((float*)x.data, (const float*)y.data, (const float*)gain.data, gather, n_gather,
@@ -1188,12 +1189,20 @@ void Ops::moe_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, con
     }
     if (rc != 3) check("moe_bf16", rc, "moe_experts(grouped)");
   }
-  took("[rows]");
+  took(rows && top > 1 ? "[rows, sums left]" : "[rows]");
   Tensor act = ws.tensor("moe.act", h.dtype, {pairs, F});
+  // one expert a token: its row is the result; else the pairs' rows, added by this call or left to the norm that reads them
+  Tensor part = top == 1 ? y : ws.tensor("moe.out", DType::F32, {pairs, W});
+  const bool left = rows && top > 1;
   int rc = KERNEL("moe", ti_moe_experts_rows)(code(h.dtype, "moe_experts"), h.data, (const int*)ids.data, (const float*)wts.data,
-                                              up.data, down.data, act.data, (float*)y.data, (int)M, (int)W, (int)F, top,
-                                              scale_input ? 1 : 0, (hipStream_t)launch_stream());
+                                              up.data, down.data, act.data, (float*)part.data, (top == 1 || left) ? nullptr : (float*)y.data,
+                                              (int)M, (int)W, (int)F, experts, top, scale_input ? 1 : 0, (hipStream_t)launch_stream());
   check("moe", rc, "moe_experts");
+  if (left) {
+    rows->t = part;
+    rows->gather = nullptr;
+    rows->n_gather = top;
+  }
 }
 
 // ----------------------------------------------------------------------------------- sampling

@@ -1513,8 +1513,9 @@ class MoE final : public FeedForwardPart {
     if (experts < 1 || experts > 1024) throw ConfigError("moe: " + std::to_string(experts) + " experts are not served (1 to 1024)");
     if (top < 1 || top > experts || top > 64)
       throw ConfigError("moe: top " + std::to_string(top) + " must lie between 1 and the number of experts (and at most 64)");
-    if (hidden * 4 > 64 * 1024)
-      throw ConfigError("moe: a width of " + std::to_string(hidden) + " is not served (a token's row must fit 64 KB)");
+    if (hidden * 4 > 64 * 1024 || intermediate * 4 > 64 * 1024)
+      throw ConfigError("moe: a width of " + std::to_string(hidden) + " / an expert size of " + std::to_string(intermediate) +
+                        " is not served (a row of either must fit 64 KB)");
     const std::string act = p.has("activation") ? p.at("activation").as_string() : "relu2";
     if (act != "relu2") throw ConfigError("moe: activation '" + act + "' is not served (only 'relu2')");
     const std::string sc = p.has("score") ? p.at("score").as_string() : "sigmoid";

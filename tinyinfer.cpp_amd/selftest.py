@@ -366,6 +366,104 @@ def case_mlstm(ops, rng, heads, dk, dv, lengths, chunk) -> int:
     return fails + _say("gated head norm", float(np.abs(_f64(out) - normed).max()), 1e-4)
 
 
+def case_norm_residual_and_experts(ops, rng) -> int:
+    """The norm onto the residual (with rows gathered on the way and a rounded copy), the router and the experts, row-wise
+    in 32-bit and bfloat16 and grouped on the matrix cores."""
+    fails = 0
+    M, H = 6, 200
+    x0, y, g = rng.normal(size=(M, H)), rng.normal(size=(9, H)) * 2, 1 + 0.2 * rng.normal(size=H)
+    gather = rng.integers(0, 9, size=(M, 2)).astype(np.int32)
+    x, copy = _dev(x0, torch.float32), torch.empty(M, H, device="cuda", dtype=torch.bfloat16)
+    ops.norm_residual(x, _dev(y, torch.float32), _dev(g, torch.float32), 1e-5, True, _dev(gather), copy)
+    yy = y[gather[:, 0]] + y[gather[:, 1]]
+    want = x0 + yy / np.sqrt((yy * yy).mean(-1, keepdims=True) + 1e-5) * g
+    fails += _say("norm onto the residual, rows gathered", float(np.abs(_f64(x) - want).max()), 5e-6)
+    fails += _say("  its rounded copy", float(np.abs(_f64(copy) - _bf16(_f64(x))).max()), 1e-12)
+    for dtype, M, W, E, top, F, tol in ((torch.float32, 7, 96, 6, 2, 80, 3e-5), (torch.bfloat16, 5, 64, 4, 3, 96, 2e-2),
+                                        (torch.bfloat16, 400, 128, 9, 2, 160, 2e-2)):
+        h = _bf16(rng.normal(size=(M, W)))
+        router = (rng.normal(size=(E, W)) * 2 / math.sqrt(W)).astype(np.float32)
+        up, down = _bf16(rng.normal(size=(E, F, W)) / math.sqrt(W)), _bf16(rng.normal(size=(E, W, F)) / math.sqrt(F))
+        ids, wts = torch.empty(M, top, device="cuda", dtype=torch.int32), torch.empty(M, top, device="cuda")
+        ops.moe_route(_dev(h, dtype), _dev(router), ids, wts, top)
+        score = 1 / (1 + np.exp(-(h @ router.astype(np.float64).T)))
+        order = np.argsort(-score, axis=1, kind="stable")[:, :top]
+        name = f"experts {top} of {E}, {M} tokens, {W} -> {F}, {str(dtype).split('.')[-1]}"
+        fails += _say(name + ": choice", float((ids.cpu().numpy() != order).sum()), 0.5)
+        out = torch.empty(M, W, device="cuda")
+        ops.moe_experts(_dev(h, dtype), ids, wts, _dev(up.reshape(E * F, W), dtype), _dev(down.reshape(E * W, F), dtype), out, E)
+        want = np.zeros((M, W))
+        for m in range(M):
+            for e in order[m]:
+                want[m] += (np.maximum((score[m, e] * h[m]) @ up[e].T, 0) ** 2) @ down[e].T
+        fails += _say(name, float(np.abs(_f64(out) - want).max() / max(1.0, np.abs(want).max())), tol)
+    return fails
+
+
+def case_diff_attention(ops, rng, nh, nkv, dk, dv, T, block, taps, rot, dtype, P=16) -> int:
+    """Short convolution, per-map norm, partial rotation and cache write in one kernel, then differential attention of every
+    row (row-wise, and for bfloat16 sizes the matrix-core kernels take: as tiles of a portion and as single tokens)."""
+    eps, lam, out_scale, scale = 1e-5, 0.7, 0.5, 1 / math.sqrt(dk)
+    C = nh * 2 * dk + nkv * (2 * dk + dv)
+    u = rng.normal(size=(T, C)).astype(np.float32)
+    tp = rng.normal(size=(C, taps)).astype(np.float32)
+    qw, kw = (1 + 0.2 * rng.normal(size=dk)).astype(np.float32), (1 + 0.2 * rng.normal(size=dk)).astype(np.float32)
+    freq = np.array([100.0 ** (-2.0 * i / max(rot, 1)) for i in range(rot // 2)], dtype=np.float32)
+    n_pages = -(-T // P)
+    table = rng.permutation(n_pages).astype(np.int32)[None, :]
+    pool = torch.zeros(n_pages, nkv, P, 2 * dk + dv, device="cuda", dtype=dtype)
+    q_out = torch.empty(T, nh * 2 * dk, device="cuda", dtype=dtype)
+    pos, slots = _dev(np.arange(T, dtype=np.int32)), _dev(np.zeros(T, dtype=np.int32))
+    state = torch.zeros(1, taps - 1, C, device="cuda")
+    entries = _dev(np.array([[0, T, 0, 0]], dtype=np.int32))
+    ops.diff_qk_prep(_dev(u), _dev(qw), _dev(kw), _dev(freq) if rot else None, None, pos, slots, _dev(table), pool, q_out, eps, nh, nkv,
+                     dk, dv, rot, 1.0, taps=_dev(tp), state=state, entries=entries)
+    pad = np.concatenate([np.zeros((taps - 1, C)), u.astype(np.float64)])
+    mixed = sum(pad[j:j + T] * tp[:, j].astype(np.float64) for j in range(taps))
+    q = mixed[:, :nh * 2 * dk].reshape(T, nh, 2, dk)
+    k = mixed[:, nh * 2 * dk: nh * 2 * dk + nkv * 2 * dk].reshape(T, nkv, 2, dk)
+    v = mixed[:, nh * 2 * dk + nkv * 2 * dk:].reshape(T, nkv, dv)
+
+    def prepare(z, w):
+        z = z / np.sqrt((z * z).mean(-1, keepdims=True) + eps) * w
+        out = z.copy()
+        for t in range(T):
+            a = np.float64(np.float32(t) * freq)
+            out[t, ..., :rot // 2] = z[t, ..., :rot // 2] * np.cos(a) - z[t, ..., rot // 2:rot] * np.sin(a)
+            out[t, ..., rot // 2:rot] = z[t, ..., rot // 2:rot] * np.cos(a) + z[t, ..., :rot // 2] * np.sin(a)
+        return out
+    rnd = _bf16 if dtype == torch.bfloat16 else (lambda t: t)
+    qn, kn, vn = rnd(prepare(q, qw)), rnd(prepare(k, kw)), rnd(v)
+    name = f"differential attention {nh}/{nkv} heads, {dk}/{dv}, {T} tokens, blocks of {block}, {taps} taps, {str(dtype).split('.')[-1]}"
+    fails = _say(name + ": q", float(np.abs(_f64(q_out).reshape(T, nh, 2, dk) - qn).max() / np.abs(qn).max()), 3e-5 if dtype == torch.float32 else 1e-2)
+    fails += _say(name + ": state left", float(np.abs(_f64(state)[0] - u[T - taps + 1:]).max()), 1e-12)
+    want = np.zeros((T, nh, dv))
+    for i in range(T):
+        lo = i // block * block
+        for h in range(nh):
+            g = h // (nh // nkv)
+            a = []
+            for mp in range(2):
+                s = (kn[lo: i + 1, g, mp] @ qn[i, h, mp]) * scale
+                p = np.exp(s - s.max())
+                a.append((p / p.sum()) @ vn[lo: i + 1, g])
+            o = a[0] - lam * a[1]
+            want[i, h] = o / math.sqrt((o * o).mean() + eps) * out_scale
+    want = want.reshape(T, -1)
+    tol = 2e-4 if dtype == torch.float32 else 3e-2
+    out = torch.empty(T, nh * dv, device="cuda", dtype=dtype)
+    args = (q_out, pool, _dev(table), pos, slots)
+    ops.diff_attention(*args, out, nh, nkv, dk, dv, scale, lam, eps, out_scale, block=block)
+    fails += _say(name, float(np.abs(_f64(out) - want).max()), tol)
+    if dtype == torch.bfloat16 and dk in (32, 64, 128) and dv in (32, 64, 128):
+        tiles = _dev(np.array([[0, r, min(64, T - r)] for r in range(0, T, 64)], dtype=np.int32))
+        ops.diff_attention(*args, out, nh, nkv, dk, dv, scale, lam, eps, out_scale, block=block, tiles=tiles, entries=entries)
+        fails += _say(name + ", tiles on the matrix cores", float(np.abs(_f64(out) - want).max()), tol)
+        ops.diff_attention(*args, out, nh, nkv, dk, dv, scale, lam, eps, out_scale, block=block, all_rows=True)
+        fails += _say(name + ", single tokens on the matrix cores", float(np.abs(_f64(out) - want).max()), tol)
+    return fails
+
+
 def run_selftest() -> int:
     if not torch.cuda.is_available():
         print("[selftest] no GPU: the kernels of this framework run on an AMD GPU (gfx950) only", flush=True)
@@ -389,6 +487,10 @@ def run_selftest() -> int:
     fails += case_capped_attention(ops, rng, nh=6, nkv=1, dk=64, dv=16, T=130, dtype=torch.bfloat16)
     fails += case_mlstm(ops, rng, heads=2, dk=32, dv=48, lengths=[150, 1, 70], chunk=64)
     fails += case_mlstm(ops, rng, heads=1, dk=128, dv=128, lengths=[200], chunk=64)
+    fails += case_norm_residual_and_experts(ops, rng)
+    fails += case_diff_attention(ops, rng, nh=3, nkv=1, dk=20, dv=12, T=90, block=37, taps=3, rot=8, dtype=torch.float32, P=8)
+    fails += case_diff_attention(ops, rng, nh=4, nkv=2, dk=32, dv=64, T=200, block=150, taps=4, rot=32, dtype=torch.bfloat16)
+    fails += case_diff_attention(ops, rng, nh=8, nkv=1, dk=64, dv=128, T=130, block=64, taps=2, rot=16, dtype=torch.bfloat16)
     fails += case_embed_argmax_sample(ops, rng)
     fails += case_model_shapes(ops, rng)
     fails += case_head_bandwidth(ops, rng)
