@@ -281,11 +281,12 @@ diff_tiles_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool,
 // ------------------------------------------------------------------------------------------ tiles, keys and values through LDS
 // The same tiles with the four wavefronts sharing what they read: a pair of blocks (32 keys: their two maps and the values)
 // is fetched once by the workgroup into one of two LDS stages while the pair before it is multiplied from the other, one
-// barrier a pair.  Key rows are padded by 16 bytes and value rows by 8, so that the fragments' reads spread over the banks.
+// barrier a pair.  Key and value rows are padded by 16 bytes, so that the fragments' reads spread over the banks; a value row
+// holds, quarter by quarter, four keys of the first block and the same four of the second: a lane's fragment in one read.
 template <int DK, int DV>
 struct DiffStage {
   static constexpr int KROW = 2 * DK + 8;       // bfloat16 elements of a key row
-  static constexpr int VROW = 32 + 4;           // of a value row: 32 keys (block A, block B)
+  static constexpr int VROW = 32 + 8;           // of a value row: per quarter q its keys 4 q .. 4 q + 3 of block A, then of block B
   static constexpr int K_ELEMS = 32 * KROW, ELEMS = K_ELEMS + DV * VROW;
   static constexpr int K_UNITS = 32 * (2 * DK / 8), V_UNITS = DV * 4;      // 16-byte pieces fetched per pair
   static constexpr int K_PER = (K_UNITS + 255) / 256, V_PER = (V_UNITS + 255) / 256;
@@ -329,10 +330,11 @@ __device__ __forceinline__ void park_pair(bf16_t* to, const uint4 (&kreg)[DiffSt
   for (int i = 0; i < S::V_PER; ++i) {
     const int u = threadIdx.x + 256 * i;
     if (S::V_UNITS % 256 == 0 || u < S::V_UNITS) {
-      const int d = u >> 2, piece = u & 3;
-      uint2* dst = reinterpret_cast<uint2*>(to + S::K_ELEMS + d * S::VROW + (piece >> 1) * 16 + (piece & 1) * 8);
-      dst[0] = make_uint2(vreg[i].x, vreg[i].y);
-      dst[1] = make_uint2(vreg[i].z, vreg[i].w);
+      // the piece holds keys 8 h .. 8 h + 7 of block `blk`: the quarters 2 h and 2 h + 1, four keys each
+      const int d = u >> 2, piece = u & 3, blk = piece >> 1, h = piece & 1;
+      bf16_t* dst = to + S::K_ELEMS + d * S::VROW + (2 * h) * 8 + blk * 4;
+      *reinterpret_cast<uint2*>(dst) = make_uint2(vreg[i].x, vreg[i].y);
+      *reinterpret_cast<uint2*>(dst + 8) = make_uint2(vreg[i].z, vreg[i].w);
     }
   }
 }
@@ -341,15 +343,19 @@ template <int DK, int DV>
 __global__ void __launch_bounds__(256)
 diff_tiles_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ pool, const int* __restrict__ table, int table_stride,
                       const int* __restrict__ tiles, const int* __restrict__ entries, bf16_t* __restrict__ out, int n_head, int n_kv,
-                      int P, float scale2, int block, int window, float lambda, float eps, float out_scale) {
+                      int P, float scale2, int block, int window, float lambda, float eps, float out_scale, int heads_per_round) {
   using S = DiffStage<DK, DV>;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   bf16_t* const lds = reinterpret_cast<bf16_t*>(lds_raw);      // two stages of S::ELEMS
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r16 = lane & 15, quad = lane >> 4;
-  const int e = tiles[3 * blockIdx.x], tile_row0 = tiles[3 * blockIdx.x + 1], tile_rows = tiles[3 * blockIdx.x + 2];
-  const int row0 = tile_row0 + 16 * wave, n_rows = tile_rows - 16 * wave;      // n_rows <= 0: a wavefront without rows (it still fetches)
+  // The tiles come from the one that walks the most keys to the one that walks the fewest, and workgroups start in the
+  // grid's order, a compute unit taking one of every `heads_per_round` heads' worth at a time: every other such group of
+  // heads walks the list backwards, so that a unit's long tile stands beside a short one.
   const int h = blockIdx.y;
+  const int t = ((h / heads_per_round) & 1) ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
+  const int e = tiles[3 * t], tile_row0 = tiles[3 * t + 1], tile_rows = tiles[3 * t + 2];
+  const int row0 = tile_row0 + 16 * wave, n_rows = tile_rows - 16 * wave;      // n_rows <= 0: a wavefront without rows (it still fetches)
   const int kvh = h / (n_head / n_kv);
   const int e_row0 = entries[4 * e], e_n = entries[4 * e + 1], e_start = entries[4 * e + 2];
   const int kv_last = e_start + e_n - 1;
@@ -431,9 +437,7 @@ diff_tiles_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ p
         }
 #pragma unroll
       for (int d = 0; d < DV / 16; ++d) {
-        const bf16_t* vr = vs + (16 * d + r16) * S::VROW + quad * 4;
-        const uint2 a = *reinterpret_cast<const uint2*>(vr), b = *reinterpret_cast<const uint2*>(vr + 16);
-        f.v[d].u = make_uint4(a.x, a.y, b.x, b.y);
+        f.v[d].u = *reinterpret_cast<const uint4*>(vs + (16 * d + r16) * S::VROW + quad * 8);
       }
       const bool plain = curA && curB && keyA >= lo_max && keyA + 31 <= hi_min;
       attend_pair<DK, DV>(f, qf, lo, hi, plain, kv_last, scale2, st);
@@ -593,13 +597,17 @@ extern "C" int ti_diff_attention_tiles_bf16(const void* q, const void* pool, con
   TI_REQUIRE(n_head <= 65535 && table_stride > 0 && block >= 0 && window >= 0, "diff_attention (tiles): bad arguments");
   if (n_tiles == 0) return 0;
   dim3 grid(n_tiles, n_head);
+  int units = 0, device = 0;
+  if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || units <= 0)
+    units = 256;
+  const int heads_per_round = units / n_tiles > 0 ? units / n_tiles : 1;
   // keys and values shared through LDS (use_lds 0: every wavefront fetches its own, for tests and measurements)
 #define DA_TILES(K, V)                                                                                                              \
   do {                                                                                                                              \
     if (use_lds)                                                                                                                    \
       diff_tiles_lds_kernel<K, V><<<grid, 256, 2 * DiffStage<K, V>::ELEMS * 2, stream>>>(                                           \
           (const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, entries, (bf16_t*)out, n_head, n_kv, page_size,        \
-          scale * DA_LOG2E, block, window, lambda, eps, out_scale);                                                                 \
+          scale * DA_LOG2E, block, window, lambda, eps, out_scale, heads_per_round);                                                \
     else                                                                                                                            \
       diff_tiles_kernel<K, V><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)pool, table, table_stride, tiles, entries, \
                                                         (bf16_t*)out, n_head, n_kv, page_size, scale * DA_LOG2E, block, window,     \
